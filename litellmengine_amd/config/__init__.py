@@ -1,6 +1,7 @@
 from .model_config import ConfigError, Qwen3Config, read_config_json, FULL_ATTENTION, SLIDING_ATTENTION
 from .visadra_config import VisadraConfig
 from .kezasun_config import KezasunConfig
+from .malilorn_config import MalilornConfig
 from .registry import (
     Architecture,
     architecture_of,
@@ -16,6 +17,7 @@ __all__ = [
     "Qwen3Config",
     "VisadraConfig",
     "KezasunConfig",
+    "MalilornConfig",
     "FULL_ATTENTION",
     "SLIDING_ATTENTION",
     "architecture_of",

@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import Block, BuildContext, Carried, Norm, Prenormed
+from ..parts.base import Block, BuildContext, Carried, Norm, Normed, Prenormed
 from ..parts.embedding import Embedding
 from ..parts.linear import Linear
 from ..weights.spec import TensorSpec
@@ -44,9 +44,12 @@ class DecoderLM:
         head: Linear,
         tied_head: bool,
         logit_scale: float = 1.0,
+        logit_softcap: Optional[float] = None,
     ):
-        """`logit_scale`: the head's result is multiplied by it (in 32-bit)."""
+        """`logit_scale`: the head's result is multiplied by it (in 32-bit).  `logit_softcap`: the
+        logits then pass through cap * tanh(logits / cap) (in 32-bit; None: not)."""
         self.logit_scale = float(logit_scale)
+        self.logit_softcap = float(logit_softcap) if logit_softcap else None
         self.config = config
         self.embedding = embedding
         self.blocks = list(blocks)
@@ -116,7 +119,10 @@ class DecoderLM:
         for i, e in enumerate(self.plan):
             # the norm that the next block starts with, if the products around it may do its work
             if i < last:
-                next_norm = self.blocks[self.plan[i + 1].block].entry_norm()
+                follower = self.blocks[self.plan[i + 1].block]
+                next_norm = follower.entry_norm()
+                if next_norm is None and self.blocks[e.block].chained_norm() is not None:
+                    next_norm = follower.chained_norm()  # (between two blocks that chain their norms)
             else:  # the final norm, where the head's product can take its place (every row goes to the head)
                 next_norm = self.final_norm if step.every_row_wanted and not self.head.has_bias else None
             delta = self.blocks[e.block].forward(hidden, delta, step, caches.layer(i), next_norm=next_norm)
@@ -124,6 +130,11 @@ class DecoderLM:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=hidden.device)
         if isinstance(delta, Carried):  # the last block has added everything into the stream itself
             delta = None
-        x = delta if isinstance(delta, Prenormed) else self.final_norm.forward(hidden, delta, rows=step.logit_rows)
+        if isinstance(delta, Normed):  # the final norm of every row, made by the last block's last launch
+            x = delta.x
+        else:
+            x = delta if isinstance(delta, Prenormed) else self.final_norm.forward(hidden, delta, rows=step.logit_rows)
         logits = self.head.forward(x, out_dtype=torch.float32)
-        return logits if self.logit_scale == 1.0 else self.ctx.ops.scale_(logits, self.logit_scale)
+        if self.logit_scale != 1.0:
+            logits = self.ctx.ops.scale_(logits, self.logit_scale)
+        return logits if self.logit_softcap is None else self.ctx.ops.softcap_(logits, self.logit_softcap)

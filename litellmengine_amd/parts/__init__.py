@@ -1,15 +1,16 @@
-from .attention import PagedAttention, SinkAttention
+from .attention import ConvAttention, PagedAttention, SinkAttention
 from .base import (Block, BuildContext, CacheField, Carried, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
                    Normed, PartialSums, PositionEncoding, Prenormed, ScaledSum, StateSpec)
-from .block import ParallelBlock, PostNormBlock, PreNormBlock
+from .block import ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock
 from .embedding import Embedding
-from .feed_forward import GatedMLP
+from .feed_forward import GatedMLP, PlainMLP
 from .latent_attention import LatentAttention
 from .linear import Linear
-from .moe import GroupLimitedMLP, RoutedMLP
+from .moe import GroupLimitedMLP, RoutedMLP, ScoreRoutedMLP
 from .norm import RMSNorm
 from .position import NoPositionEncoding, RotaryHalfSplit, RotaryInterleaved
 from .recurrent import MinGRU
+from .side_by_side import SideBySideMixer
 from .wkv import WKVMixer
 
 __all__ = [
@@ -17,4 +18,5 @@ __all__ = [
     "RoutedMLP", "RotaryInterleaved", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
     "NoPositionEncoding", "Norm", "NormFold", "Normed", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec", "GroupLimitedMLP", "ParallelBlock", "ScaledSum", "SinkAttention", "WKVMixer",
+    "ConvAttention", "SandwichBlock", "PlainMLP", "ScoreRoutedMLP", "SideBySideMixer",
 ]

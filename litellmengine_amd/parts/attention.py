@@ -20,7 +20,8 @@ import torch
 
 from ..csrc.limits import check_head_dim
 from ..weights.spec import INIT_NORM, INIT_NORMAL, TensorSpec
-from .base import BuildContext, CacheSpec, KVCacheSpec, Mixer, PositionEncoding
+from ..weights.spec import INIT_WIDE
+from .base import BuildContext, CacheSpec, KVCacheSpec, Mixer, PositionEncoding, StateSpec
 from .linear import Linear
 
 
@@ -240,3 +241,105 @@ class SinkAttention(Mixer):
                                 sinks=self.sinks)
         gated = ops.head_gate(a, qkvg, qkvg.shape[1] - self.nq, self.nq, self.vdim)
         return self.o.forward(gated)
+
+
+class ConvAttention(Mixer):
+    """Grouped-query attention whose projections pass a short causal convolution over time first:
+
+        u = (W_q h, W_k h, W_v h)                         one stacked product, no biases
+        c_t = sum_j taps[:, j] * u_(t - J + 1 + j)        per channel, J taps, zeros before a request's start
+        q, k <- every head of c's q and k parts divided by its root mean square, times one weight [dim]
+                for all heads; then the position encoding on the first elements of every head
+        p_j = softmax_j((q . k_j) * scale) over every earlier token and the token itself
+        out = out_scale * W_o [heads' sum_j p_j v_j]
+
+    Keys may be `dim` wide and values `vdim`: the cache's heads hold `cache_dim` >= both elements (a
+    multiple of 32, which the matrix-core kernels take), the rest zeros, so the kernels of
+    `PagedAttention` serve; the output projection reads zeros against zero columns there.  The last
+    J - 1 rows of u of every request are its state (`StateSpec`, float32): what the next step's first
+    tokens are convolved with.  The taps are kept in 32-bit, and `out_scale` is folded into the taps of
+    v (the result is linear in v), so it costs no operation and no rounding of its own."""
+
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden_size: int, num_q_heads: int, num_kv_heads: int, dim: int, vdim: int,
+                 position: PositionEncoding, norm_eps: float, scale: float, taps: int = 0, out_scale: float = 1.0,
+                 names: Sequence[str] = ("q", "k", "v", "o"), conv_suffix: str = ".conv", norm_suffix: str = ".norm"):
+        """`taps`: the convolution's length J (0 or 1 without a tensor: none).  The checkpoint's tensors are
+        `prefix` + q, k, v (projections), + `conv_suffix` (their taps, [channels, J]), + `norm_suffix` (q and k: the
+        heads' norm weight [dim]) and o."""
+        if num_q_heads % num_kv_heads:
+            raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+        self.cache_dim = -(-max(dim, vdim) // 32) * 32
+        check_head_dim(self.cache_dim, getattr(position, "rotary_dim", 0))
+        if getattr(position, "rotary_dim", 0) > dim:
+            raise ValueError("the rotation covers more elements than a key has")
+        if taps < 0:
+            raise ValueError("a convolution has no negative number of taps")
+        self.prefix, self.hidden = prefix, hidden_size
+        self.nq, self.nkv, self.dim, self.vdim = num_q_heads, num_kv_heads, dim, vdim
+        self.position = position
+        self.eps, self.scale, self.out_scale = float(norm_eps), float(scale), float(out_scale)
+        self.taps = int(taps)
+        q, k, v, o = (prefix + n for n in names)
+        self.proj_names = (q, k, v)
+        self.widths = (num_q_heads * dim, num_kv_heads * dim, num_kv_heads * vdim)
+        self.cols = sum(self.widths)
+        self.conv_suffix, self.norm_suffix = conv_suffix, norm_suffix
+        self.o_name = o
+        self.o = Linear([o], num_q_heads * vdim, [hidden_size])
+        self.weight = self.conv_w = self.q_norm_w = self.k_norm_w = None
+
+    @property
+    def kept_rows(self) -> int:
+        """Rows of the projections that a request keeps from step to step."""
+        return max(0, self.taps - 1)
+
+    def cache_spec(self) -> CacheSpec:
+        return KVCacheSpec(self.nkv, self.cache_dim, None)
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return StateSpec((self.kept_rows * self.cols,), torch.float32) if self.kept_rows else None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = dict(self.o.tensor_specs())
+        for name, rows in zip(self.proj_names, self.widths):
+            specs[name] = TensorSpec((rows, self.hidden), INIT_NORMAL)
+            if self.taps:
+                specs[name + self.conv_suffix] = TensorSpec((rows, self.taps), INIT_WIDE)
+        for name in self.proj_names[:2]:
+            specs[name + self.norm_suffix] = TensorSpec((self.dim,), INIT_NORM)
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.position.bind(weights, ctx)
+        self.weight = torch.cat([weights[n].to(ctx.dtype) for n in self.proj_names], dim=0).contiguous()
+        if self.taps:
+            taps = torch.cat([weights[n + self.conv_suffix].float() for n in self.proj_names], dim=0)
+        else:  # one tap of one: the projection itself
+            taps = torch.ones((self.cols, 1), dtype=torch.float32, device=self.weight.device)
+        taps = taps.clone()
+        taps[self.widths[0] + self.widths[1]:] *= self.out_scale  # the attention's result is linear in v
+        self.conv_w = taps.to(ctx.device).contiguous()
+        self.q_norm_w = weights[self.proj_names[0] + self.norm_suffix].float().contiguous()
+        self.k_norm_w = weights[self.proj_names[1] + self.norm_suffix].float().contiguous()
+        o = weights[self.o_name].to(ctx.dtype)
+        if self.cache_dim != self.vdim:  # the attention hands out heads of cache_dim elements, zeros past vdim
+            o = torch.nn.functional.pad(o.view(self.hidden, self.nq, self.vdim), (0, self.cache_dim - self.vdim))
+            o = o.reshape(self.hidden, self.nq * self.cache_dim)
+        self.o.bind_tensor(o.contiguous(), ctx)
+
+    def forward(self, x, step, cache):
+        ops = self.ctx.ops
+        group = cache.group
+        u = ops.linear(x, self.weight)
+        cos_sin, rot = self.position.fused_rotary(step)
+        q = ops.conv_norm_rope_write(u, self.conv_w, cache.state if self.kept_rows else None, step.token_seq,
+                                     step.cu_tokens, step.seq_slots, group.slot_mapping, self.q_norm_w, self.k_norm_w,
+                                     cos_sin, rot, self.eps, cache.kv, self.nq, self.nkv, self.dim, self.vdim, cache.writes)
+        if self.kept_rows:
+            ops.conv_state_update(u, cache.state, self.kept_rows, step.cu_tokens, step.seq_slots)
+        a = ops.paged_attention(q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens,
+                                step.token_seq, None, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len)
+        return self.o.forward(a)

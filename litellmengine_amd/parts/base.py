@@ -201,10 +201,13 @@ class Norm(Part):
     def of_embedding(self, ids: torch.Tensor, table: torch.Tensor, step=None):
         return None
 
-    def add_normed(self, hidden: torch.Tensor, y: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def add_normed(self, hidden: torch.Tensor, y: torch.Tensor, extra: Optional[torch.Tensor] = None,
+                   then: Optional["Norm"] = None) -> torch.Tensor:
         """For arrangements that norm a sublayer's OUTPUT: hidden += norm(y [+ extra]) in 32-bit, in
         place; returns the new rows of `hidden` in the activation type.  `y` and `extra` are
-        [N, width], each in the activation type or in 32-bit."""
+        [N, width], each in the activation type or in 32-bit.  With `then` (the norm that reads the
+        stream next) the return value is then.forward(hidden, None) instead: that norm of the new rows,
+        from the same launch where the two norms have a kernel for it."""
         raise NotImplementedError
 
     def fold(self, hidden: torch.Tensor) -> Optional[NormFold]:
@@ -280,6 +283,12 @@ class Block(Part):
     mixer: Mixer
 
     def entry_norm(self) -> Optional[Norm]:
+        return None
+
+    def chained_norm(self) -> Optional[Norm]:
+        """The norm of the residual stream that the block begins with, if the block takes its result
+        ready-made (a `Normed` for `delta`) from a block before it that adds into the stream itself
+        and can norm the new rows in the same launch; the model passes it to that block as `next_norm`."""
         return None
 
     def input_norm(self) -> Optional[Norm]:

@@ -147,3 +147,66 @@ class ParallelBlock(Block):
         a = self.mixer.forward(h, step, cache)
         b = self.feed_forward.forward(h) if self.feed_forward is not None else None
         return ScaledSum(a, b, self.mult)
+
+
+class SandwichBlock(Block):
+    """Residual block with a norm before and a norm after each sublayer:
+        x <- x + norm_mix_out(mixer(norm_in(x)));  x <- x + norm_ff_out(ff(norm_ff_in(x)))
+    The norm after a sublayer is applied by a kernel that also adds its result into the 32-bit
+    stream, and where the norms have a kernel for it, that launch norms the new rows for whoever
+    reads them next (`Norm.add_normed(..., then=)`): the feed-forward's norm, the next block's first
+    norm (`next_norm`; the block then returns a `Normed`), so every sublayer costs one norm launch.
+    A sublayer may hand its result on as a pair whose sum is meant (two mixers side by side, a routed
+    feed-forward with a shared expert): the norm's kernel adds the two.  A block without a feed-forward
+    is the first line alone."""
+
+    def __init__(self, norm_in: Norm, mixer: Mixer, norm_mix_out: Norm, norm_ff_in: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None, norm_ff_out: Optional[Norm] = None):
+        if not ((norm_ff_in is None) == (feed_forward is None) == (norm_ff_out is None)):
+            raise ValueError("a feed-forward and its two norms come together")
+        self.norm_in, self.mixer, self.norm_mix_out = norm_in, mixer, norm_mix_out
+        self.norm_ff_in, self.feed_forward, self.norm_ff_out = norm_ff_in, feed_forward, norm_ff_out
+
+    def _parts(self):
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_mix_out, self.norm_ff_in, self.feed_forward,
+                                 self.norm_ff_out) if p is not None)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for p in self._parts():
+            specs.update(p.tensor_specs())
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        for p in self._parts():
+            p.bind(weights, ctx)
+
+    def input_norm(self):
+        return self.norm_in
+
+    def chained_norm(self):
+        return self.norm_in
+
+    @staticmethod
+    def _pair(y):
+        return y if isinstance(y, tuple) else (y, None)
+
+    def forward(self, hidden, delta, step, cache, next_norm=None):
+        if isinstance(delta, Carried):  # the block before has added everything into the stream itself
+            delta = None
+        if isinstance(delta, Prenormed):
+            raise ValueError("a block with norms on both sides of its sublayers takes no folded norm")
+        x = delta.x if isinstance(delta, Normed) else self.norm_in.forward(hidden, delta)
+        y, extra = self._pair(self.mixer.forward(x, step, cache))
+        if self.feed_forward is None:
+            if next_norm is None:
+                self.norm_mix_out.add_normed(hidden, y, extra)
+                return None
+            return Normed(self.norm_mix_out.add_normed(hidden, y, extra, then=next_norm))
+        x = self.norm_mix_out.add_normed(hidden, y, extra, then=self.norm_ff_in)
+        y, extra = self._pair(self.feed_forward.forward(x))
+        if next_norm is None:
+            self.norm_ff_out.add_normed(hidden, y, extra)
+            return None
+        return Normed(self.norm_ff_out.add_normed(hidden, y, extra, then=next_norm))

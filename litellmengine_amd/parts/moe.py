@@ -19,7 +19,7 @@ import torch
 
 from ..weights.spec import INIT_NORMAL, TensorSpec
 from .base import BuildContext, FeedForward
-from .feed_forward import GatedMLP
+from .feed_forward import GatedMLP, PlainMLP
 from .linear import Linear
 
 
@@ -123,3 +123,58 @@ class GroupLimitedMLP(FeedForward):
         logits = self.router.forward(x, out_dtype=torch.float32)
         ids, gains = ops.moe_route_grouped(logits, self.correction, self.top, self.groups, self.groups_kept)
         return ops.moe_experts(x, ids, gains, self.gate_up, self.down)  # float32 [N, hidden]; ids from E on: x itself
+
+
+class ScoreRoutedMLP(FeedForward):
+    """Mixture of experts whose router scores every expert on its own and weighs the experts' INPUTS:
+
+        s = sigmoid(W_router h)                        32-bit
+        chosen = the `top` largest s (the lower index wins a tie); their weights are s itself, not renormalised
+        out = sum_k expert_k(s_k * h) + sigmoid(w_sg . h) * shared(h),   expert(x) = down(act(up x)), act = relu squared
+
+    The experts have no gate and no biases; their weights are stacked, the choice stays on the device.  A weight on
+    an expert's input is a factor on its first product's result, where the kernels apply it in 32-bit before the
+    activation.  The shared expert (None: none) has the same form and one gate number per token, which comes out of
+    the router's product (its row is stacked under the router's).  The routed sum is left in 32-bit; with a shared
+    expert the result is the pair (routed sum, gated shared result), which the norm's kernel adds up."""
+
+    def __init__(self, prefix: str, hidden_size: int, expert_size: int, num_experts: int, top: int,
+                 shared: Optional[PlainMLP] = None, shared_gate_name: str = "shared.sg", expert_prefix: str = "e{}.",
+                 names=("up", "down"), router_name: str = "router"):
+        if not 0 < top <= num_experts:
+            raise ValueError("every token uses between one and all of the experts")
+        self.prefix, self.hidden, self.ff, self.E, self.top = prefix, hidden_size, expert_size, num_experts, top
+        self.shared = shared
+        self.expert_names = [[prefix + expert_prefix.format(e) + n for n in names] for e in range(num_experts)]
+        rows, sizes = [prefix + router_name], [num_experts]
+        if shared is not None:
+            rows.append(prefix + shared_gate_name)
+            sizes.append(1)
+        self.router = Linear(rows, hidden_size, sizes)
+        self.up = self.down = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = dict(self.router.tensor_specs())
+        for up, down in self.expert_names:
+            specs[up] = TensorSpec((self.ff, self.hidden), INIT_NORMAL)
+            specs[down] = TensorSpec((self.hidden, self.ff), INIT_NORMAL)
+        if self.shared is not None:
+            specs.update(self.shared.tensor_specs())
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.router.bind(weights, ctx)
+        self.up = torch.stack([weights[u].to(ctx.dtype) for u, _ in self.expert_names]).contiguous()  # [E, ff, hidden]
+        self.down = torch.stack([weights[d].to(ctx.dtype) for _, d in self.expert_names]).contiguous()  # [E, hidden, ff]
+        if self.shared is not None:
+            self.shared.bind(weights, ctx)
+
+    def forward(self, x):
+        ops = self.ctx.ops
+        logits = self.router.forward(x, out_dtype=torch.float32)  # [N, E (+ 1: the shared expert's gate)]
+        ids, gains = ops.moe_route(logits, None, self.top, score="sigmoid", experts=self.E)
+        routed = ops.moe_experts(x, ids, gains, self.up, self.down, form="relu2", gain_on_input=True)  # float32 [N, hidden]
+        if self.shared is None:
+            return routed
+        return routed, self.shared.forward(x, row_gate=(logits, self.E))

@@ -33,8 +33,14 @@ class RMSNorm(Norm):
             w = 1.0 + w.float()
         self.weight = (w.reshape(1).expand(self.size) if self.scalar else w).contiguous()
 
-    def add_normed(self, hidden, y, extra=None) -> torch.Tensor:
-        return self.ctx.ops.rmsnorm_add(hidden, y, self.weight, self.eps, self.ctx.dtype, extra)
+    def add_normed(self, hidden, y, extra=None, then=None) -> torch.Tensor:
+        ops = self.ctx.ops
+        if then is None:
+            return ops.rmsnorm_add(hidden, y, self.weight, self.eps, self.ctx.dtype, extra)
+        if isinstance(then, RMSNorm) and then.size == self.size:  # both norms in one launch
+            return ops.rmsnorm_add_rmsnorm(hidden, y, self.weight, self.eps, then.weight, then.eps, self.ctx.dtype, extra)
+        ops.rmsnorm_add(hidden, y, self.weight, self.eps, self.ctx.dtype, extra)
+        return then.forward(hidden, None)
 
     def forward(self, hidden, delta, rows=None) -> torch.Tensor:
         if isinstance(delta, ScaledSum):  # the add, times its constant, and the norm in one launch

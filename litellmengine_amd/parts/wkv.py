@@ -34,8 +34,10 @@ class WKVMixer(Mixer):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, heads: int, dim: int, decay_rank: int, norm_eps: float,
-                 names: Sequence[str] = ("r", "k", "v", "g", "w1", "w2", "w0", "u", "norm", "o"), mu_prefix: str = "mu."):
-        """`names`: the checkpoint's names after `prefix` of the four input projections, the decay's two
+                 names: Sequence[str] = ("r", "k", "v", "g", "w1", "w2", "w0", "u", "norm", "o"), mu_prefix: str = "mu.",
+                 out_scale: float = 1.0):
+        """`out_scale`: the result is multiplied by it; it is folded into the 32-bit output norm's weight, so it
+        costs no operation and no rounding of its own.  `names`: the checkpoint's names after `prefix` of the four input projections, the decay's two
         projections and its offset, the bonus, the output norm's weight and the output projection; the mixing
         weights are `mu_prefix` + r, k, v, g, w."""
         if not 0 < dim <= MAX_HEAD_CHANNELS:
@@ -44,6 +46,7 @@ class WKVMixer(Mixer):
             raise ValueError("the decay's inner rank must be positive")
         self.prefix, self.hidden, self.H, self.dim, self.rank = prefix, hidden_size, heads, dim, int(decay_rank)
         self.eps = float(norm_eps)
+        self.out_scale = float(out_scale)
         r, k, v, g, w1, w2, w0, u, norm, o = (prefix + n for n in names)
         hd = heads * dim
         self.r, self.k, self.v, self.g = (Linear([n], hidden_size, [hd]) for n in (r, k, v, g))
@@ -75,7 +78,7 @@ class WKVMixer(Mixer):
         self.mu = torch.stack([weights[n].float() for n in self.mu_names]).contiguous()
         self.w0 = weights[self.w0_name].float().reshape(-1).contiguous()
         self.u = weights[self.u_name].float().reshape(-1).contiguous()
-        self.norm_w = weights[self.norm_name].float().contiguous()
+        self.norm_w = (weights[self.norm_name].float() * self.out_scale).contiguous()
 
     def forward(self, x, step, cache):
         ops = self.ctx.ops

@@ -17,7 +17,7 @@ from typing import Dict, Mapping
 import torch
 
 from .loader import WEIGHTS_FILE
-from .spec import INIT_NORM, INIT_NORMAL, TensorSpec
+from .spec import INIT_NORM, INIT_NORMAL, INIT_WIDE, TensorSpec
 
 
 def _seed_of(seed: int, name: str) -> int:
@@ -31,6 +31,8 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, dtype: torch.dtype, de
         raise ValueError(f"{name}: no random rule for integer tables")
     if spec.init == INIT_NORMAL:
         t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, 0.02, generator=gen)
+    elif spec.init == INIT_WIDE:
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, 0.5, generator=gen)
     elif spec.init == INIT_NORM:
         t = torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(-0.1, 0.1, generator=gen) + 1.0
     else:

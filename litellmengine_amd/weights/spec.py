@@ -7,6 +7,7 @@ from typing import Tuple
 # how the random-weights mode fills a tensor
 INIT_NORMAL = "normal"  # N(0, 0.02): projections, embedding tables
 INIT_NORM = "norm"  # 1 + U(-0.1, 0.1): norm weights
+INIT_WIDE = "wide"  # N(0, 0.5): the few taps of a short convolution
 
 
 @dataclasses.dataclass(frozen=True)

@@ -263,10 +263,15 @@ class TorchOps:
         return out.to(out_dtype)
 
     # -- routed feed-forward -----------------------------------------------------------------
-    def moe_route(self, logits, bias, top):
-        v = logits.to(self.cd) + bias.to(self.cd)
-        vals, idx = torch.topk(v, top, dim=-1)
-        return idx.to(torch.int32), torch.softmax(vals, dim=-1).to(torch.float32)
+    def moe_route(self, logits, bias, top, score="softmax_chosen", experts=None):
+        v = logits.to(self.cd)[:, : experts or logits.shape[1]]
+        if bias is not None:
+            v = v + bias.to(self.cd)
+        # (a stable sort: among equal values the lower index comes first)
+        idx = torch.sort(v, dim=-1, descending=True, stable=True).indices[:, :top]
+        vals = torch.gather(v, 1, idx)
+        gains = torch.sigmoid(vals) if score == "sigmoid" else torch.softmax(vals, dim=-1)
+        return idx.to(torch.int32), gains.to(torch.float32)
 
     def moe_route_grouped(self, logits, correction, top, groups=1, keep=1):
         s = torch.softmax(logits.to(self.cd), dim=-1)
@@ -282,7 +287,9 @@ class TorchOps:
         chosen = torch.gather(s, 1, ids)
         return ids.to(torch.int32), (chosen / (chosen.sum(-1, keepdim=True) + 1e-20)).to(torch.float32)
 
-    def moe_experts(self, x, ids, gains, gate_up, down):
+    def moe_experts(self, x, ids, gains, gate_up, down, form="gated_silu", gain_on_input=False):
+        if form != "gated_silu" or gain_on_input:
+            return self._moe_experts_plain(x, ids, gains, gate_up, down, form, gain_on_input)
         N, top = ids.shape
         ff = gate_up.shape[1] // 2
         out = torch.zeros((N, down.shape[1]), dtype=self.cd, device=x.device)
@@ -298,6 +305,106 @@ class TorchOps:
                 a = a.to(x.dtype).to(self.cd)
                 out[n] += gains[n, k].to(self.cd) * (down[e].to(self.cd) @ a)
         return out.to(torch.float32)
+
+    def _moe_experts_plain(self, x, ids, gains, up, down, form, gain_on_input):
+        assert form == "relu2"
+        N, top = ids.shape
+        out = torch.zeros((N, down.shape[1]), dtype=self.cd, device=x.device)
+        xx = x.to(self.cd)
+        for n in range(N):
+            for k in range(top):
+                e, g = int(ids[n, k]), gains[n, k].to(self.cd)
+                z = up[e].to(self.cd) @ xx[n]
+                if gain_on_input:
+                    z = z * g
+                a = (torch.clamp(z, min=0.0) ** 2).to(x.dtype).to(self.cd)
+                y = down[e].to(self.cd) @ a
+                out[n] += y if gain_on_input else g * y
+        return out.to(torch.float32)
+
+    def bias_act(self, z, kind, gated, bias=None, row_gate=None):
+        zz = z.to(self.cd)
+        if bias is not None:
+            zz = zz + bias.to(self.cd)
+        act = {"silu": lambda t: t * torch.sigmoid(t), "relu": lambda t: torch.clamp(t, min=0.0),
+               "relu2": lambda t: torch.clamp(t, min=0.0) ** 2}[kind]
+        if gated:
+            F = zz.shape[1] // 2
+            out = act(zz[:, :F]) * zz[:, F:]
+        else:
+            out = act(zz)
+        if row_gate is not None:
+            t, col = row_gate
+            out = out * torch.sigmoid(t[:, col].to(self.cd))[:, None]
+        return out.to(z.dtype)
+
+    def softcap_(self, x, cap):
+        x.copy_((cap * torch.tanh(x.to(self.cd) / cap)).to(x.dtype))
+        return x
+
+    def rmsnorm_add_rmsnorm(self, hidden, y, weight, eps, next_weight, next_eps, out_dtype, extra=None):
+        self.rmsnorm_add(hidden, y, weight, eps, out_dtype, extra)
+        x = hidden.to(self.cd)
+        return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + next_eps) * next_weight.to(self.cd)).to(out_dtype)
+
+    # -- attention behind a short convolution ------------------------------------------------------
+    def conv_norm_rope_write(self, u, taps, state, token_seq, cu_tokens, seq_slots, slots, q_weight, k_weight, cos_sin,
+                             rotary_dim, eps, kv_layer, num_q_heads, num_kv_heads, dim, vdim, write_kv=True):
+        nq, nkv = num_q_heads, num_kv_heads
+        N, cols = u.shape
+        J = taps.shape[1]
+        D, P = kv_layer.shape[4], kv_layer.shape[3]
+        uu, tt = u.to(self.cd), taps.to(self.cd)
+        c = torch.zeros_like(uu)
+        for s in range(seq_slots.shape[0]):
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 <= q0:
+                continue
+            if J > 1:
+                before = state[int(seq_slots[s]), : (J - 1) * cols].to(self.cd).view(J - 1, cols)
+                rows = torch.cat([before, uu[q0:q1]], dim=0)
+            else:
+                rows = uu[q0:q1]
+            for j in range(J):
+                c[q0:q1] += rows[j : j + (q1 - q0)] * tt[:, j]
+
+        def norm(t, w):
+            return t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps) * w.to(self.cd)
+
+        def rope(t):
+            if rotary_dim == 0:
+                return t
+            half = rotary_dim // 2
+            co, si = cos_sin[:, None, :, 0].to(self.cd), cos_sin[:, None, :, 1].to(self.cd)
+            x1, x2 = t[..., :half], t[..., half:rotary_dim]
+            return torch.cat([x1 * co - x2 * si, x2 * co + x1 * si, t[..., rotary_dim:]], dim=-1)
+
+        def padded(t):
+            return torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+
+        qw, kw = nq * dim, nkv * dim
+        q = padded(rope(norm(c[:, :qw].reshape(N, nq, dim), q_weight)))
+        if write_kv:
+            k = padded(rope(norm(c[:, qw : qw + kw].reshape(N, nkv, dim), k_weight)))
+            v = padded(c[:, qw + kw : qw + kw + nkv * vdim].reshape(N, nkv, vdim))
+            for n in range(N):
+                slot = int(slots[n])
+                if slot < 0:
+                    continue
+                page, off = slot // P, slot % P
+                kv_layer[page, 0, :, off, :] = k[n].to(kv_layer.dtype)
+                v_pages(kv_layer)[page, :, :, off] = v[n].to(kv_layer.dtype)
+        return q.to(u.dtype).contiguous()
+
+    def conv_state_update(self, u, state, kept, cu_tokens, seq_slots):
+        cols = u.shape[1]
+        for s in range(seq_slots.shape[0]):
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 <= q0:
+                continue
+            slot = int(seq_slots[s])
+            rows = torch.cat([state[slot, : kept * cols].view(kept, cols), u[q0:q1].to(state.dtype)], dim=0)
+            state[slot, : kept * cols] = rows[-kept:].reshape(-1)
 
     # -- projections normed as a whole, gates per head, side-by-side sublayers -------------------
     def proj_norm_rope_write(self, qkv, bias, slots, q_weight, k_weight, cos_sin, rotary_dim, eps, kv_layer,
