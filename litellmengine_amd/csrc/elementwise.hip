@@ -219,3 +219,70 @@ extern "C" int lle_tanh(void* x, int64_t total, int dtype, hipStream_t stream) {
     else tanh_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)x, total);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------
+// Activations of feed-forwards that the fused silu product does not cover.
+//   gated:  out[n, f] = act(z[n, f] + b[f]) * (z[n, F + f] + b[F + f])        z [N, 2 F]
+//   plain:  out[n, f] = act(z[n, f] + b[f])                                   z [N, F]
+// times sigmoid(row_gate[n * gate_stride + gate_col]) where a row gate is given (float32).
+// act: 0 silu, 1 relu, 2 the square of relu.  `b` may be null.  Everything in 32-bit.
+// ---------------------------------------------------------------------------------
+#define LLE_ACT_SILU 0
+#define LLE_ACT_RELU 1
+#define LLE_ACT_RELU2 2
+
+__device__ __forceinline__ float apply_act(float x, int kind) {
+    if (kind == LLE_ACT_SILU) return x / (1.0f + expf(-x));
+    const float r = fmaxf(x, 0.f);
+    return kind == LLE_ACT_RELU ? r : r * r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_act_kernel(const T* __restrict__ z, const T* __restrict__ bias,
+                                                        const float* __restrict__ row_gate, int gate_stride, int gate_col,
+                                                        T* __restrict__ out, int N, int F, int gated, int kind) {
+    const int64_t total = (int64_t)N * F;
+    const int in_cols = gated ? 2 * F : F;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t n = idx / F;
+        const int f = (int)(idx - n * F);
+        const T* row = z + n * in_cols;
+        float a = apply_act(to_f32<T>(row[f]) + (bias ? to_f32<T>(bias[f]) : 0.f), kind);
+        if (gated) a *= to_f32<T>(row[F + f]) + (bias ? to_f32<T>(bias[F + f]) : 0.f);
+        if (row_gate) a *= 1.0f / (1.0f + expf(-row_gate[n * gate_stride + gate_col]));
+        out[idx] = from_f32<T>(a);
+    }
+}
+
+extern "C" int lle_bias_act(const void* z, const void* bias, const void* row_gate, int gate_stride, int gate_col,
+                            void* out, int N, int F, int gated, int kind, int dtype, hipStream_t stream) {
+    if (N <= 0 || F <= 0) return 0;
+    if (kind < 0 || kind > LLE_ACT_RELU2) return (int)hipErrorInvalidValue;
+    int64_t blocks = ((int64_t)N * F + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == LLE_F32)
+        bias_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)z, (const float*)bias, (const float*)row_gate,
+                                                                 gate_stride, gate_col, (float*)out, N, F, gated, kind);
+    else
+        bias_act_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)z, (const bf16_t*)bias,
+                                                                  (const float*)row_gate, gate_stride, gate_col,
+                                                                  (bf16_t*)out, N, F, gated, kind);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// x = cap * tanh(x / cap), float32, in place
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, int64_t total, float cap) {
+    const float inv = 1.0f / cap;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x)
+        x[idx] = cap * tanhf(x[idx] * inv);
+}
+extern "C" int lle_softcap(void* x, int64_t total, float cap, hipStream_t stream) {
+    if (total <= 0) return 0;
+    if (!(cap > 0.f)) return (int)hipErrorInvalidValue;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    softcap_kernel<<<(int)blocks, 256, 0, stream>>>((float*)x, total, cap);
+    LLE_RETURN_LAUNCH_STATUS();
+}

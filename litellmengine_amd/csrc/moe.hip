@@ -22,13 +22,16 @@ LLE_DEFINE_ERROR_STRING()
 // one wavefront per token: the `top` largest of logits + bias (the lower index wins a tie), then the softmax
 // over those alone.  ids int32 [N, top], gains float32 [N, top].  Every round each lane looks through its own
 // experts (lane, lane + 64, ...) for the best one not chosen yet, and the wavefront picks the best of the lanes.
+// `bias` may be null; a row of `logits` holds `stride` >= E numbers, of which the first E are the experts'.
+// mode 0: gains = softmax over the chosen alone; mode 1: gains = sigmoid of every chosen value, as it is.
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
                                                          const float* __restrict__ bias, int32_t* __restrict__ ids,
-                                                         float* __restrict__ gains, int N, int E, int top) {
+                                                         float* __restrict__ gains, int N, int E, int top, int stride,
+                                                         int mode) {
     const int n = blockIdx.x * (blockDim.x / LLE_WAVE) + threadIdx.x / LLE_WAVE;
     const int lane = threadIdx.x % LLE_WAVE;
     if (n >= N) return;  // (the whole wavefront)
-    const float* row = logits + (int64_t)n * E;
+    const float* row = logits + (int64_t)n * stride;
     int chosen[MOE_MAX_TOP];   // the same in every lane
     float value[MOE_MAX_TOP];
     for (int k = 0; k < top; ++k) {
@@ -37,7 +40,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         for (int e = lane; e < E; e += LLE_WAVE) {
             bool taken = false;
             for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
-            const float v = row[e] + bias[e];
+            const float v = row[e] + (bias ? bias[e] : 0.f);
             if (!taken && (best == 0x7fffffff || v > bv)) {  // (e rises: an equal value later loses)
                 best = e;
                 bv = v;
@@ -56,6 +59,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         value[k] = bv;
     }
     if (lane != 0) return;
+    if (mode == 1) {
+        for (int k = 0; k < top; ++k) {
+            ids[(int64_t)n * top + k] = chosen[k];
+            gains[(int64_t)n * top + k] = 1.0f / (1.0f + expf(-value[k]));
+        }
+        return;
+    }
     float sum = 0.f;
     const float largest = value[0];
     for (int k = 0; k < top; ++k) {
@@ -69,11 +79,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 }
 
 extern "C" int lle_moe_route(const void* logits, const void* bias, void* ids, void* gains, int N, int E, int top,
-                             hipStream_t stream) {
+                             int stride, int mode, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (top <= 0 || top > MOE_MAX_TOP || top > E) return (int)hipErrorInvalidValue;
+    if (top <= 0 || top > MOE_MAX_TOP || top > E || stride < E || mode < 0 || mode > 1) return (int)hipErrorInvalidValue;
     moe_route_kernel<<<(N + 3) / 4, 256, 0, stream>>>((const float*)logits, (const float*)bias, (int32_t*)ids,
-                                                           (float*)gains, N, E, top);
+                                                           (float*)gains, N, E, top, stride, mode);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -196,20 +206,40 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __re
     return wave_sum(acc);
 }
 
+// The experts' form.  MOE_GATED_SILU: act = silu(Wg x) * (Wu x), weights [E, 2 F, K] (gate rows, then up rows).
+// MOE_PLAIN_RELU2: act = relu(Wu x)^2, weights [E, F, K].  `in_gains` (or null): the pair's gain multiplies the
+// expert's INPUT, which is a factor on its first products' results; it is applied there, in 32-bit, before the
+// activation (the gain then takes no part in the sum of the experts' results).
+#define MOE_GATED_SILU 0
+#define MOE_PLAIN_RELU2 1
+
+__device__ __forceinline__ float moe_relu2(float z) {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+}
+
 // grid (pairs, ceil(F / 4)), 4 wavefronts: wavefront w makes act[p, f], f = 4 blockIdx.y + w
-template <typename T>
+template <typename T, int FORM>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids,
-                                                           const T* __restrict__ gate_up, T* __restrict__ act, int top,
-                                                           int F, int K, int E) {
+                                                           const T* __restrict__ gate_up,
+                                                           const float* __restrict__ in_gains, T* __restrict__ act,
+                                                           int top, int F, int K, int E) {
     const int p = blockIdx.x;
     const int f = blockIdx.y * 4 + threadIdx.x / LLE_WAVE;
     if (f >= F) return;
     const int e = ids[p];
     if (e >= E) return;  // an identity expert: nothing to multiply
     const T* xr = x + (int64_t)(p / top) * K;
+    const float gain = in_gains ? in_gains[p] : 1.0f;
+    if (FORM == MOE_PLAIN_RELU2) {
+        const T* w = gate_up + (int64_t)e * F * K;
+        const float z = gain * wave_dot<T>(xr, w + (int64_t)f * K, K);
+        if (threadIdx.x % LLE_WAVE == 0) act[(int64_t)p * F + f] = from_f32<T>(moe_relu2(z));
+        return;
+    }
     const T* w = gate_up + (int64_t)e * 2 * F * K;
-    const float g = wave_dot<T>(xr, w + (int64_t)f * K, K);
-    const float u = wave_dot<T>(xr, w + (int64_t)(F + f) * K, K);
+    const float g = gain * wave_dot<T>(xr, w + (int64_t)f * K, K);
+    const float u = gain * wave_dot<T>(xr, w + (int64_t)(F + f) * K, K);
     if (threadIdx.x % LLE_WAVE == 0) act[(int64_t)p * F + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
 }
 
@@ -226,36 +256,47 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
     for (int k = 0; k < top; ++k) {
         const int p = n * top + k;
         const int e = ids[p];
+        const float gain = gains ? gains[p] : 1.0f;  // (no gains: they entered with the experts' inputs)
         if (e >= E) {  // (the same for the whole wavefront)
-            total += gains[p] * to_f32<T>(x[(int64_t)n * H + o]);
+            total += gain * to_f32<T>(x[(int64_t)n * H + o]);
             continue;
         }
         const T* w = down + ((int64_t)e * H + o) * F;
-        total += gains[p] * wave_dot<T>(act + (int64_t)p * F, w, F);
+        total += gain * wave_dot<T>(act + (int64_t)p * F, w, F);
     }
     if (threadIdx.x % LLE_WAVE == 0) out[(int64_t)n * H + o] = total;
 }
 
-// x [N, K], ids/gains [N, top], gate_up [E, 2 F, K], down [E, H, F], act [N top, F] (scratch), out float32 [N, H];
-// ids from E on are identity experts (then H = K)
+template <typename T>
+static void moe_experts_pairs(const void* x, const void* ids, const void* gains, const void* gate_up, const void* down,
+                              void* act, void* out, int N, int top, int E, int F, int K, int H, int form,
+                              int gain_on_input, hipStream_t stream) {
+    const dim3 g1(N * top, (F + 3) / 4), g2(N, (H + 3) / 4);
+    const float* in_gains = gain_on_input ? (const float*)gains : nullptr;
+    const float* out_gains = gain_on_input ? nullptr : (const float*)gains;
+    if (form == MOE_PLAIN_RELU2)
+        moe_gate_up_kernel<T, MOE_PLAIN_RELU2><<<g1, 256, 0, stream>>>((const T*)x, (const int32_t*)ids,
+                                                                         (const T*)gate_up, in_gains, (T*)act, top, F, K, E);
+    else
+        moe_gate_up_kernel<T, MOE_GATED_SILU><<<g1, 256, 0, stream>>>((const T*)x, (const int32_t*)ids,
+                                                                        (const T*)gate_up, in_gains, (T*)act, top, F, K, E);
+    moe_down_kernel<T><<<g2, 256, 0, stream>>>((const T*)act, (const int32_t*)ids, out_gains, (const T*)down,
+                                                (const T*)x, (float*)out, top, F, H, E);
+}
+
+// x [N, K], ids/gains [N, top], gate_up [E, 2 F, K] (form 0) or [E, F, K] (form 1), down [E, H, F], act [N top, F]
+// (scratch), out float32 [N, H]; ids from E on are identity experts (then H = K); `gain_on_input`: the gains
+// multiply the experts' inputs, not their results
 extern "C" int lle_moe_experts(const void* x, const void* ids, const void* gains, const void* gate_up,
                                const void* down, void* act, void* out, int N, int top, int E, int F, int K, int H,
-                               int dtype, hipStream_t stream) {
+                               int dtype, int form, int gain_on_input, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (top <= 0 || (int64_t)N * top > 0x7fffffff) return (int)hipErrorInvalidValue;
-    const dim3 g1(N * top, (F + 3) / 4), g2(N, (H + 3) / 4);
-    if (g1.y > 65535 || g2.y > 65535) return (int)hipErrorInvalidValue;
-    if (dtype == LLE_F32) {
-        moe_gate_up_kernel<float><<<g1, 256, 0, stream>>>((const float*)x, (const int32_t*)ids, (const float*)gate_up,
-                                                           (float*)act, top, F, K, E);
-        moe_down_kernel<float><<<g2, 256, 0, stream>>>((const float*)act, (const int32_t*)ids, (const float*)gains,
-                                                        (const float*)down, (const float*)x, (float*)out, top, F, H, E);
-    } else {
-        moe_gate_up_kernel<bf16_t><<<g1, 256, 0, stream>>>((const bf16_t*)x, (const int32_t*)ids,
-                                                            (const bf16_t*)gate_up, (bf16_t*)act, top, F, K, E);
-        moe_down_kernel<bf16_t><<<g2, 256, 0, stream>>>((const bf16_t*)act, (const int32_t*)ids, (const float*)gains,
-                                                         (const bf16_t*)down, (const bf16_t*)x, (float*)out, top, F, H, E);
-    }
+    if (top <= 0 || (int64_t)N * top > 0x7fffffff || form < 0 || form > 1) return (int)hipErrorInvalidValue;
+    if ((F + 3) / 4 > 65535 || (H + 3) / 4 > 65535) return (int)hipErrorInvalidValue;
+    if (dtype == LLE_F32)
+        moe_experts_pairs<float>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, stream);
+    else
+        moe_experts_pairs<bf16_t>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, stream);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -421,11 +462,15 @@ __device__ __forceinline__ bool moe_find_tile(const int32_t* __restrict__ plan, 
     return true;
 }
 
-// act[row, f] = silu(x Wg^T) * (x Wu^T) for the sorted rows; items (tile, block of 128 f), 4 wavefronts of 32 f each
+// act[row, f] = silu(x Wg^T) * (x Wu^T) for the sorted rows; items (tile, block of 128 f), 4 wavefronts of 32 f each.
+// FORM MOE_PLAIN_RELU2: act[row, f] = relu(x Wu^T)^2; items (tile, block of 256 f), 4 wavefronts of 64 f each.
+// `in_gains` (or null): a pair's gain as a factor on its products' results, before the activation.
+template <int FORM>
 __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* __restrict__ x,
                                                                 const int32_t* __restrict__ plan,
                                                                 const int32_t* __restrict__ order,
                                                                 const bf16_t* __restrict__ gate_up,
+                                                                const float* __restrict__ in_gains,
                                                                 bf16_t* __restrict__ act, int E, int top, int F, int K,
                                                                 int tiles, int blocks) {
     MoeTile t;
@@ -433,19 +478,25 @@ __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* 
     if (!moe_grid_item(tiles, blocks, tile, block) || !moe_find_tile(plan, E, tile, t)) return;
     __shared__ __attribute__((aligned(16))) bf16_t s_x[2][MOE_TM][MOE_XS];
     const int lane = threadIdx.x % LLE_WAVE, c = lane / 16, r = lane % 16;
-    const int f0 = (block * 4 + threadIdx.x / LLE_WAVE) * 32;  // (a wavefront past F multiplies zeros: it shares the barriers)
+    const int per_wave = FORM == MOE_PLAIN_RELU2 ? 64 : 32;
+    const int f0 = (block * 4 + threadIdx.x / LLE_WAVE) * per_wave;  // (a wavefront past F multiplies zeros: it shares the barriers)
     const bf16_t* xrow[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int row = threadIdx.x / 4 + 64 * j;
         xrow[j] = row < t.rows ? x + (int64_t)(order[t.row0 + row] / top) * K : nullptr;
     }
-    const bf16_t* w = gate_up + (int64_t)t.expert * 2 * F * K;
-    const bf16_t* wr[4];  // gate rows f0 + r, f0 + 16 + r, then the up rows of the same f
+    const bf16_t* w = gate_up + (int64_t)t.expert * (FORM == MOE_PLAIN_RELU2 ? 1 : 2) * F * K;
+    const bf16_t* wr[4];  // gate rows f0 + r, f0 + 16 + r, then the up rows of the same f; plain: four tiles of up rows
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
-        const int f = f0 + (nt % 2) * 16 + r;
-        wr[nt] = f < F ? w + (int64_t)((nt / 2) * F + f) * K : nullptr;
+        if (FORM == MOE_PLAIN_RELU2) {
+            const int f = f0 + nt * 16 + r;
+            wr[nt] = f < F ? w + (int64_t)f * K : nullptr;
+        } else {
+            const int f = f0 + (nt % 2) * 16 + r;
+            wr[nt] = f < F ? w + (int64_t)((nt / 2) * F + f) * K : nullptr;
+        }
     }
     mf32x4 acc[4][8];
 #pragma unroll
@@ -457,6 +508,19 @@ __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* 
     for (int mt = 0; mt < 8; ++mt) {
         const int row = mt * 16 + r;
         if (row >= t.rows) continue;
+        const float gain = in_gains ? in_gains[order[t.row0 + row]] : 1.0f;
+        if (FORM == MOE_PLAIN_RELU2) {
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const int f = f0 + nt * 16 + 4 * c;
+                if (f >= F) continue;  // (F is a multiple of 4: whole groups)
+                mbf16x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = (bf16_t)moe_relu2(gain * acc[nt][mt][i]);
+                *(mbf16x4*)(act + (int64_t)(t.row0 + row) * F + f) = v;
+            }
+            continue;
+        }
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const int f = f0 + half * 16 + 4 * c;
@@ -464,7 +528,7 @@ __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* 
             mbf16x4 v;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float g = acc[half][mt][i], u = acc[2 + half][mt][i];
+                const float g = gain * acc[half][mt][i], u = gain * acc[2 + half][mt][i];
                 v[i] = (bf16_t)(g / (1.0f + expf(-g)) * u);
             }
             *(mbf16x4*)(act + (int64_t)(t.row0 + row) * F + f) = v;
@@ -523,11 +587,12 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const float* __restrict
         mf32x4 total = mf32x4{0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < top; ++k) {
             const int p = n * top + k;
+            const float gain = gains ? gains[p] : 1.0f;  // (no gains: they entered with the experts' inputs)
             if (place[p] < 0) {
                 const mbf16x4 xv = *(const mbf16x4*)(x + (int64_t)n * H + o);
-                total += gains[p] * mf32x4{(float)xv[0], (float)xv[1], (float)xv[2], (float)xv[3]};
+                total += gain * mf32x4{(float)xv[0], (float)xv[1], (float)xv[2], (float)xv[3]};
             } else {
-                total += gains[p] * *(const mf32x4*)(y + (int64_t)place[p] * H + o);
+                total += gain * *(const mf32x4*)(y + (int64_t)place[p] * H + o);
             }
         }
         *(mf32x4*)(out + (int64_t)n * H + o) = total;
@@ -540,10 +605,14 @@ extern "C" int lle_moe_tile_rows(void) { return MOE_TM; }
 // place int32 [N top], act bfloat16 [N top, F], y float32 [N top, H].
 extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void* gains, const void* gate_up,
                                      const void* down, void* plan, void* order, void* place, void* act, void* y,
-                                     void* out, int N, int top, int E, int F, int K, int H, hipStream_t stream) {
+                                     void* out, int N, int top, int E, int F, int K, int H, int form, int gain_on_input,
+                                     hipStream_t stream) {
     if (N <= 0) return 0;
     const int64_t pairs64 = (int64_t)N * top;
-    if (top <= 0 || E <= 0 || E > 256 || K % 8 || F % 8 || H % 4 || pairs64 > 0x3fffffff) return (int)hipErrorInvalidValue;
+    if (top <= 0 || E <= 0 || E > 256 || K % 8 || F % 8 || H % 4 || pairs64 > 0x3fffffff || form < 0 || form > 1)
+        return (int)hipErrorInvalidValue;
+    const float* in_gains = gain_on_input ? (const float*)gains : nullptr;
+    const float* out_gains = gain_on_input ? nullptr : (const float*)gains;
     const int pairs = (int)pairs64;
     const int tiles = pairs / MOE_TM + E;  // at most: every expert leaves one tile partly empty
     moe_zero_kernel<<<(2 * E + 255) / 256, 256, 0, stream>>>((int32_t*)plan, 2 * E);
@@ -551,13 +620,18 @@ extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void*
     moe_plan_kernel<<<1, 256, 0, stream>>>((int32_t*)plan, E);
     moe_place_kernel<<<(pairs + 255) / 256, 256, 0, stream>>>((const int32_t*)ids, (int32_t*)plan, (int32_t*)order,
                                                                (int32_t*)place, pairs, E);
-    const int fb = (F + 127) / 128, hb = (H + 255) / 256;
-    moe_gate_up_tile_kernel<<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
-        (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, (bf16_t*)act, E, top, F, K,
-        tiles, fb);
+    const int fb = form == MOE_PLAIN_RELU2 ? (F + 255) / 256 : (F + 127) / 128, hb = (H + 255) / 256;
+    if (form == MOE_PLAIN_RELU2)
+        moe_gate_up_tile_kernel<MOE_PLAIN_RELU2><<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
+            (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, in_gains, (bf16_t*)act,
+            E, top, F, K, tiles, fb);
+    else
+        moe_gate_up_tile_kernel<MOE_GATED_SILU><<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
+            (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, in_gains, (bf16_t*)act,
+            E, top, F, K, tiles, fb);
     moe_down_tile_kernel<<<8 * ((tiles * hb + 7) / 8), 256, 0, stream>>>(
         (const bf16_t*)act, (const int32_t*)plan, (const bf16_t*)down, (float*)y, E, F, H, tiles, hb);
-    moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, (const float*)gains,
+    moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, out_gains,
                                                 (const bf16_t*)x, (float*)out, top, H);
     LLE_RETURN_LAUNCH_STATUS();
 }

@@ -451,3 +451,87 @@ extern "C" int lle_scaled_add_rmsnorm(void* hidden, const void* a, int a_dtype, 
                                                                   eps);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------
+// Two norms around one add, for arrangements with a norm after a sublayer and a norm before the next:
+//   hidden += RMSNorm(y [+ extra]) * w_out        (32-bit, in place)
+//   out     = RMSNorm(hidden) * w_next            (the new row's norm, in the activation type)
+// One workgroup a row; a thread keeps its share of the row (up to NR_PER elements) in registers from
+// the first sum to the last store, so y, extra and hidden are read once.  Rows wider than
+// NR_PER * threads take the plain loops.
+// ---------------------------------------------------------------------------------
+#define NR_PER 8
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void rmsnorm_add_rmsnorm_kernel(
+    float* __restrict__ hidden, const void* __restrict__ y, int y_dtype, const void* __restrict__ extra, int extra_dtype,
+    const void* __restrict__ w_out, const void* __restrict__ w_next, int weight_dtype, TO* __restrict__ out, int H,
+    float eps_out, float eps_next) {
+    __shared__ float red[16];
+    const int64_t at = (int64_t)blockIdx.x * H;
+    if (H <= NR_PER * (int)blockDim.x) {
+        float v[NR_PER];
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NR_PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            v[j] = 0.f;
+            if (i < H) {
+                v[j] = load_as_f32(y, at + i, y_dtype);
+                if (extra) v[j] += load_as_f32(extra, at + i, extra_dtype);
+            }
+            ss += v[j] * v[j];
+        }
+        const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_out);
+        ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NR_PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < H) {
+                v[j] = hidden[at + i] + v[j] * inv * load_as_f32(w_out, i, weight_dtype);
+                hidden[at + i] = v[j];
+                ss += v[j] * v[j];
+            }
+        }
+        const float inv2 = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_next);
+#pragma unroll
+        for (int j = 0; j < NR_PER; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < H) out[at + i] = from_f32<TO>(v[j] * inv2 * load_as_f32(w_next, i, weight_dtype));
+        }
+        return;
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = load_as_f32(y, at + i, y_dtype);
+        if (extra) v += load_as_f32(extra, at + i, extra_dtype);
+        ss += v * v;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_out);
+    ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = load_as_f32(y, at + i, y_dtype);
+        if (extra) v += load_as_f32(extra, at + i, extra_dtype);
+        const float h = hidden[at + i] + v * inv * load_as_f32(w_out, i, weight_dtype);
+        hidden[at + i] = h;
+        ss += h * h;
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps_next);
+    for (int i = threadIdx.x; i < H; i += blockDim.x)  // (every thread reads back what it wrote itself)
+        out[at + i] = from_f32<TO>(hidden[at + i] * inv2 * load_as_f32(w_next, i, weight_dtype));
+}
+
+// both weights have the same type
+extern "C" int lle_rmsnorm_add_rmsnorm(void* hidden, const void* y, int y_dtype, const void* extra, int extra_dtype,
+                                       const void* w_out, const void* w_next, int weight_dtype, void* out, int R, int H,
+                                       float eps_out, float eps_next, int out_dtype, hipStream_t stream) {
+    if (R <= 0) return 0;
+    const int threads = H > 4096 ? 1024 : H > 2048 ? 512 : 256;
+    if (out_dtype == LLE_F32)
+        rmsnorm_add_rmsnorm_kernel<float><<<R, threads, 0, stream>>>((float*)hidden, y, y_dtype, extra, extra_dtype, w_out,
+                                                                      w_next, weight_dtype, (float*)out, H, eps_out, eps_next);
+    else
+        rmsnorm_add_rmsnorm_kernel<bf16_t><<<R, threads, 0, stream>>>((float*)hidden, y, y_dtype, extra, extra_dtype, w_out,
+                                                                       w_next, weight_dtype, (bf16_t*)out, H, eps_out, eps_next);
+    LLE_RETURN_LAUNCH_STATUS();
+}

@@ -53,6 +53,16 @@ def _dev(t: torch.Tensor, name: str, dtype=None) -> None:
         raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
 
 
+def _rows(t: torch.Tensor, name: str, dtype=None) -> None:
+    """A matrix whose rows may lie apart (some columns of a wider one): elements of a row are neighbours."""
+    if not t.is_cuda:
+        raise KernelError(f"{name} must live on the GPU")
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name} must be a matrix with contiguous rows")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
+
+
 # the current stream's handle without the Stream object around it (a launch is a few microseconds
 # of Python as it is; torch.cuda.current_stream() alone costs as much again)
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -893,17 +903,23 @@ class HipOps:
         return out
 
     # -- routed feed-forward ----------------------------------------------------------
-    def moe_route(self, logits, bias, top: int):
-        """float32 logits [N, E] + bias [E] -> (int32 ids [N, top] of the largest, the lower index first
-        among equals; float32 gains [N, top]: the softmax over the chosen alone)."""
+    def moe_route(self, logits, bias, top: int, score: str = "softmax_chosen", experts: Optional[int] = None):
+        """float32 logits [N, >= E] (+ bias [E], or None) -> (int32 ids [N, top] of the largest among the first
+        E = `experts` columns (default: all), the lower index first among equals; float32 gains [N, top]).
+        `score`: "softmax_chosen": the softmax over the chosen alone; "sigmoid": the sigmoid of every chosen
+        value, as it is."""
         _dev(logits, "router logits", torch.float32)
-        _dev(bias, "router bias", torch.float32)
-        N, E = logits.shape
-        _need(bias.shape == (E,) and 0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
+        N, cols = logits.shape
+        E = cols if experts is None else int(experts)
+        _need(0 < E <= cols and 0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
+        _need(score in ("softmax_chosen", "sigmoid"), f"unknown router score {score!r}")
+        if bias is not None:
+            _dev(bias, "router bias", torch.float32)
+            _need(bias.shape == (E,), "the router's bias must be [E]")
         ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
         gains = torch.empty((N, top), dtype=torch.float32, device=logits.device)
-        self._run("moe", "lle_moe_route", [_P, _P, _P, _P, _I, _I, _I, _P], _ptr(logits), _ptr(bias), _ptr(ids),
-                  _ptr(gains), N, E, top)
+        self._run("moe", "lle_moe_route", [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _ptr(logits), _ptr(bias), _ptr(ids),
+                  _ptr(gains), N, E, top, cols, 1 if score == "sigmoid" else 0)
         return ids, gains
 
     def moe_route_grouped(self, logits, correction, top: int, groups: int = 1, keep: int = 1):
@@ -926,10 +942,13 @@ class HipOps:
 
     MOE_TILED_MIN_PAIRS = 129  # (token, choice) pairs from which the sorted, tiled kernels take a bfloat16 step
 
-    def moe_experts(self, x, ids, gains, gate_up, down) -> torch.Tensor:
+    def moe_experts(self, x, ids, gains, gate_up, down, form: str = "gated_silu", gain_on_input: bool = False) -> torch.Tensor:
         """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
         float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].  An id from E on
         names an identity expert, whose result is x itself (then H = K).
+        `form` "relu2": experts without a gate, down[e] relu(up[e] x)^2, `gate_up` is up [E, F, K].
+        `gain_on_input`: the result is sum_k expert_e(gains[n, k] * x) instead; the gain is applied to the first
+        products' results, in 32-bit, before the activation.
         Few pairs, or float32: every pair streams its expert's rows.  Many bfloat16 pairs: sorted by expert
         on the device, then tiles of 128 pairs of one expert on the matrix cores."""
         _dev(x, "x")
@@ -939,25 +958,29 @@ class HipOps:
         _dev(down, "down", x.dtype)
         N, K = x.shape
         top = ids.shape[1]
+        _need(form in ("gated_silu", "relu2"), f"unknown expert form {form!r}")
+        plain = form == "relu2"
         E, F2, _ = gate_up.shape
         H = down.shape[1]
+        F = F2 if plain else F2 // 2
         _need(ids.shape == (N, top) and gains.shape == (N, top), "ids and gains must be [N, top]")
-        _need(gate_up.shape == (E, F2, K) and F2 % 2 == 0 and down.shape == (E, H, F2 // 2), "expert weights do not fit")
-        act = torch.empty((N * top, F2 // 2), dtype=x.dtype, device=x.device)
+        _need(gate_up.shape == (E, F2, K) and (plain or F2 % 2 == 0) and down.shape == (E, H, F), "expert weights do not fit")
+        act = torch.empty((N * top, F), dtype=x.dtype, device=x.device)
         out = torch.empty((N, H), dtype=torch.float32, device=x.device)
-        F = F2 // 2
+        code, on_input = (1 if plain else 0), (1 if gain_on_input else 0)
         if (x.dtype == torch.bfloat16 and N * top >= self.MOE_TILED_MIN_PAIRS and E <= 256 and K % 8 == 0 and F % 8 == 0
                 and H % 4 == 0):
             plan = torch.empty((4 * E + 1,), dtype=torch.int32, device=x.device)
             order = torch.empty((2, N * top), dtype=torch.int32, device=x.device)
             y = torch.empty((N * top, H), dtype=torch.float32, device=x.device)
-            self._run("moe", "lle_moe_experts_tiled", [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+            self._run("moe", "lle_moe_experts_tiled",
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
                       _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(plan), order[0].data_ptr(),
-                      order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H)
+                      order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H, code, on_input)
             return out
-        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-                  _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, E, F2 // 2,
-                  K, H, dtype_code(x.dtype))
+        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+                  _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, E, F,
+                  K, H, dtype_code(x.dtype), code, on_input)
         return out
 
     # -- projections normed as a whole, sinks' attention gates -------------------------------
@@ -1050,7 +1073,7 @@ class HipOps:
         token of a request's portion state[slot, prev_offset : prev_offset + W] (float32; what the step before
         left there).  mu float32 [M, W]."""
         _dev(x, "x")
-        _dev(state, "state", torch.float32)
+        _rows(state, "state", torch.float32)
         _dev(mu, "mu", torch.float32)
         for t, name in ((token_seq, "token_seq"), (cu_tokens, "cu_tokens"), (seq_slots, "seq_slots")):
             _dev(t, name, torch.int32)
@@ -1075,8 +1098,9 @@ class HipOps:
         `out_dtype`.  The last row of every request's x [N, W] is saved behind the matrix state.
         `max_q_len` (a host-side bound) only decides into how many pieces a walk is cut."""
         HD = heads * dim
-        for t, name in ((r, "r"), (k, "k"), (v, "v"), (wraw, "wraw"), (w0, "w0"), (u, "u"), (state, "state")):
+        for t, name in ((r, "r"), (k, "k"), (v, "v"), (wraw, "wraw"), (w0, "w0"), (u, "u")):
             _dev(t, name, torch.float32)
+        _rows(state, "state", torch.float32)
         _dev(g, "g", out_dtype)
         _dev(x, "x", out_dtype)
         _dev(norm_w, "norm weight")
@@ -1104,6 +1128,123 @@ class HipOps:
                   dtype_code(norm_w.dtype), float(eps), _ptr(x), _ptr(state), state.stride(0), HD * dim, _ptr(seq_slots),
                   _ptr(cu_tokens), _ptr(out), S, heads, dim, W, pieces, piece, _ptr(part), dtype_code(out_dtype))
         return out
+
+    # -- activations, caps, chained norms ---------------------------------------------------------
+    ACT_CODES = {"silu": 0, "relu": 1, "relu2": 2}
+
+    def bias_act(self, z, kind: str, gated: bool, bias=None, row_gate=None) -> torch.Tensor:
+        """gated: z [N, 2 F] (gate columns first) -> act(gate + b) * (up + b), [N, F]; else z [N, F] -> act(z + b).
+        `kind`: silu, relu, relu2 (the square of relu); `bias` (or None) covers z's row; `row_gate` = (t, col), t
+        float32 [N, any]: row n is multiplied by sigmoid(t[n, col]).  Everything in 32-bit."""
+        _dev(z, "z")
+        _need(kind in self.ACT_CODES, f"unknown activation {kind!r}")
+        N, cols = z.shape
+        _need(not gated or cols % 2 == 0, "a gated input has an even width")
+        F = cols // 2 if gated else cols
+        if bias is not None:
+            _dev(bias, "bias", z.dtype)
+            _need(bias.shape == (cols,), "bias must cover the whole row")
+        gate_t, stride, col = None, 0, 0
+        if row_gate is not None:
+            gate_t, col = row_gate
+            _dev(gate_t, "row gate", torch.float32)
+            _need(gate_t.dim() == 2 and gate_t.shape[0] == N and 0 <= col < gate_t.shape[1], "row gate [N, > col]")
+            stride = gate_t.shape[1]
+        out = torch.empty((N, F), dtype=z.dtype, device=z.device)
+        self._run("elementwise", "lle_bias_act", [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _P], _ptr(z), _ptr(bias),
+                  _ptr(gate_t), stride, int(col), _ptr(out), N, F, 1 if gated else 0, self.ACT_CODES[kind],
+                  dtype_code(z.dtype))
+        return out
+
+    def softcap_(self, x, cap: float) -> torch.Tensor:
+        """float32 x = cap * tanh(x / cap), in place."""
+        _dev(x, "x", torch.float32)
+        _need(cap > 0.0, "a cap must be positive")
+        self._run("elementwise", "lle_softcap", [_P, _L, _F, _P], _ptr(x), x.numel(), float(cap))
+        return x
+
+    def rmsnorm_add_rmsnorm(self, hidden, y, weight, eps: float, next_weight, next_eps: float, out_dtype,
+                            extra=None) -> torch.Tensor:
+        """hidden float32 [N, H] += RMSNorm(y [+ extra]) * weight, in place and in 32-bit; returns
+        RMSNorm(the new hidden) * next_weight in `out_dtype`: the norm after one sublayer and the norm before
+        the next in one launch.  `y`, `extra`: [N, H], float32 or bfloat16 each."""
+        _dev(hidden, "hidden", torch.float32)
+        _dev(weight, "norm weight")
+        _dev(next_weight, "next norm weight", weight.dtype)
+        N, H = hidden.shape
+        _need(weight.shape == (H,) and next_weight.shape == (H,), f"norm weights must be [{H}]")
+        for t, name in ((y, "y"), (extra, "extra")):
+            if t is not None:
+                _dev(t, name)
+                _need(t.shape == hidden.shape, f"{name} must have the shape of hidden")
+        out = torch.empty((N, H), dtype=out_dtype, device=hidden.device)
+        self._run("norm", "lle_rmsnorm_add_rmsnorm", [_P, _P, _I, _P, _I, _P, _P, _I, _P, _I, _I, _F, _F, _I, _P],
+                  _ptr(hidden), _ptr(y), dtype_code(y.dtype), _ptr(extra), dtype_code(extra.dtype) if extra is not None else 0,
+                  _ptr(weight), _ptr(next_weight), dtype_code(weight.dtype), _ptr(out), N, H, float(eps), float(next_eps),
+                  dtype_code(out_dtype))
+        return out
+
+    # -- attention behind a short convolution --------------------------------------------------------
+    def conv_norm_rope_write(self, u, taps, state, token_seq, cu_tokens, seq_slots, slots, q_weight, k_weight, cos_sin,
+                             rotary_dim: int, eps: float, kv_layer, num_q_heads: int, num_kv_heads: int, dim: int,
+                             vdim: int, write_kv: bool = True) -> torch.Tensor:
+        """A row of u holds q [nq dim], k [nkv dim], v [nkv vdim] of one token.  Every channel is convolved over
+        time with its J taps (float32 [cols, J]; the last tap meets the token itself), reading the rows of the
+        same request ahead of it in this step and, before those, the request's state row (float32
+        [slots + 1, (J - 1) cols], the last J - 1 rows of u that earlier steps brought, oldest first; None for
+        J = 1).  Then every head of q and k is divided by its root mean square times q_weight / k_weight
+        (float32 [dim], one for all heads), the first `rotary_dim` elements of every head are rotated (half-split)
+        by cos_sin [N, rotary_dim / 2, 2].  Returns q [N, nq, D], D = kv_layer.shape[4] >= max(dim, vdim), zeros
+        past dim; K and V^T go to the pages at `slots` with zeros past dim and vdim.  The state is left as it
+        is: conv_state_update advances it."""
+        _dev(u, "u")
+        _dev(taps, "taps", torch.float32)
+        _dev(slots, "slots", torch.int32)
+        _dev(kv_layer, "kv_layer", u.dtype)
+        for t, name in ((token_seq, "token_seq"), (cu_tokens, "cu_tokens"), (seq_slots, "seq_slots")):
+            _dev(t, name, torch.int32)
+        nq, nkv = num_q_heads, num_kv_heads
+        N, cols = u.shape
+        J = taps.shape[1]
+        S = seq_slots.shape[0]
+        _need(cols == (nq + nkv) * dim + nkv * vdim, "a row of u holds q, k and v")
+        _need(taps.shape == (cols, J) and J >= 1, "taps must be [cols, J]")
+        _need(slots.shape == (N,) and token_seq.shape == (N,) and cu_tokens.shape == (S + 1,), "slots, token_seq [N]; cu_tokens [S + 1]")
+        _need(kv_layer.dim() == 5 and kv_layer.shape[1] == 2 and kv_layer.shape[2] == nkv, "kv_layer must be [pages, 2, nkv, page_size, D]")
+        D, page_size = kv_layer.shape[4], kv_layer.shape[3]
+        _need(D >= max(dim, vdim), "the cache's heads are smaller than the model's")
+        _need(0 <= rotary_dim <= dim and rotary_dim % 2 == 0, "rotary_dim must be even and <= dim")
+        if J > 1:
+            _need(state is not None, "a convolution of several taps needs the requests' state rows")
+            _rows(state, "state", torch.float32)
+            _need(state.shape[1] >= (J - 1) * cols, "a state row holds J - 1 rows of u")
+        _dev(q_weight, "q norm weight", torch.float32)
+        _dev(k_weight, "k norm weight", torch.float32)
+        _need(q_weight.shape == (dim,) and k_weight.shape == (dim,), f"the heads' norm weights must be [{dim}]")
+        if rotary_dim > 0:
+            _dev(cos_sin, "cos_sin", torch.float32)
+            _need(cos_sin.shape == (N, rotary_dim // 2, 2), "cos_sin must be [N, rotary_dim / 2, 2]")
+        q_out = torch.empty((N, nq, D), dtype=u.dtype, device=u.device)
+        self._run("rope_kv", "lle_conv_norm_rope_write",
+                  [_P, _I, _P, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _I, _I, _P],
+                  _ptr(u), cols, _ptr(taps), J, _ptr(state) if J > 1 else None, state.stride(0) if J > 1 else 0,
+                  _ptr(token_seq), _ptr(cu_tokens), _ptr(seq_slots), _ptr(slots), _ptr(q_weight), _ptr(k_weight),
+                  _ptr(cos_sin) if rotary_dim > 0 else None, rotary_dim, float(eps), _ptr(q_out), _ptr(kv_layer), N, nq, nkv,
+                  dim, vdim, D, page_size, kv_layer.stride(0), 1 if write_kv else 0, dtype_code(u.dtype))
+        return q_out
+
+    def conv_state_update(self, u, state, kept: int, cu_tokens, seq_slots) -> None:
+        """state row of every request of the step <- the last `kept` rows of (the `kept` rows it held, then the
+        request's rows of u in this step); state float32 [slots + 1, >= kept * cols], u [N, cols]."""
+        _dev(u, "u")
+        _rows(state, "state", torch.float32)
+        _dev(cu_tokens, "cu_tokens", torch.int32)
+        _dev(seq_slots, "seq_slots", torch.int32)
+        N, cols = u.shape
+        S = seq_slots.shape[0]
+        _need(kept > 0 and state.shape[1] >= kept * cols and cu_tokens.shape == (S + 1,), "a state row holds `kept` rows of u")
+        self._run("rope_kv", "lle_conv_state_update", [_P, _I, _P, _L, _I, _P, _P, _I, _I, _P], _ptr(u), cols, _ptr(state),
+                  state.stride(0), int(kept), _ptr(cu_tokens), _ptr(seq_slots), S, dtype_code(u.dtype))
 
     # -- picking tokens --------------------------------------------------------------
     def argmax(self, logits, scatter=None) -> torch.Tensor:

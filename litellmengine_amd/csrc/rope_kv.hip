@@ -502,3 +502,160 @@ extern "C" int lle_proj_norm_rope_write(const void* qkv, int cols, const void* b
             page_stride, has_kv, write_kv);
     LLE_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------
+// Projections behind a short causal convolution over time.  A row of `u` holds q [nq dim], k [nkv dim]
+// and v [nkv vdim] of one token.  Per channel c and token t of a request,
+//     conv_t[c] = sum_j taps[c, j] * u_(t - J + 1 + j)[c]          taps float32 [cols, J]
+// where a row before the portion that this step brings comes from the request's state row (the last
+// J - 1 rows of u of the steps before, oldest first, float32; zeros at a request's start) and rows before
+// the request's start are zeros by that.  Then every head of q and k is divided by its root mean square
+// times one weight [dim] for all heads, the first `rot` elements of every head are rotated in the half-split
+// layout, q leaves as [N, nq, D] (zeros past dim) and K, V^T go to the pages with zeros past dim and vdim.
+// grid = tokens, a wavefront of the workgroup per head, four heads at a time; all arithmetic in 32-bit.
+// The state is advanced by conv_state_kernel, a launch of its own behind this one (every token of a
+// portion reads the rows that the step found there).
+// ---------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float conv_at(const T* __restrict__ u, int cols, const float* __restrict__ taps, int J,
+                                         const float* __restrict__ kept, int64_t n, int before, int c) {
+    // `before`: rows of this request in this step ahead of row n; kept: [J - 1, cols] or null
+    float acc = 0.f;
+    for (int j = 0; j < J; ++j) {
+        const int back = J - 1 - j;  // how many tokens back this tap reaches
+        float x;
+        if (back <= before)
+            x = to_f32<T>(u[(n - back) * cols + c]);
+        else
+            x = kept ? kept[(int64_t)(J - 1 - (back - before)) * cols + c] : 0.f;
+        acc += taps[(int64_t)c * J + j] * x;
+    }
+    return acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
+    const T* __restrict__ u, int cols, const float* __restrict__ taps, int J, const float* __restrict__ state,
+    int64_t state_stride, const int32_t* __restrict__ token_seq, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ slots, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, const float* __restrict__ cos_sin, int rot, float eps, T* __restrict__ q_out,
+    T* __restrict__ kv_layer, int nq, int nkv, int dim, int vdim, int D, int page_size, int64_t page_stride,
+    int write_kv) {
+    extern __shared__ float conv_row[];  // the token's convolved q and k heads, one head per wavefront at a time
+    const int64_t n = blockIdx.x;
+    const int seq = token_seq[n];
+    const int before = (int)(n - cu_tokens[seq]);
+    const float* kept = (state && J > 1) ? state + (int64_t)seq_slots[seq] * state_stride : nullptr;
+    const float* cs = cos_sin + n * rot;  // [rot / 2][2]
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE, waves = blockDim.x / LLE_WAVE;
+    float* mine = conv_row + (int64_t)wave * dim;
+    const int slot = slots[n];
+    const bool writes = write_kv && slot >= 0;
+    const int page = writes ? slot / page_size : 0, off = writes ? slot - page * page_size : 0;
+    T* dst = kv_layer + (int64_t)page * page_stride;
+    const int half = rot / 2;
+    const int heads = nq + (writes ? nkv : 0);
+    for (int h0 = 0; h0 < heads; h0 += waves) {  // (the same number of rounds for every wavefront: barriers inside)
+        const int h = h0 + wave;
+        const bool active = h < heads;
+        const bool is_q = h < nq;
+        const int col0 = is_q ? h * dim : nq * dim + (h - nq) * dim;
+        const float* w = is_q ? q_weight : k_weight;
+        float ss = 0.f;
+        if (active)
+            for (int e = lane; e < dim; e += LLE_WAVE) {
+                const float x = conv_at<T>(u, cols, taps, J, kept, n, before, col0 + e);
+                mine[e] = x;
+                ss += x * x;
+            }
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+        __syncthreads();
+        if (active)
+            for (int e = lane; e < D; e += LLE_WAVE) {
+                float y = 0.f;
+                if (e < dim) {
+                    y = mine[e] * inv * w[e];
+                    if (e < rot) {
+                        const bool low = e < half;
+                        const int i = low ? e : e - half;
+                        const int pe = low ? e + half : e - half;
+                        const float p = mine[pe] * inv * w[pe];
+                        const float c = cs[2 * i], s = cs[2 * i + 1];
+                        y = low ? y * c - p * s : y * c + p * s;
+                    }
+                }
+                if (is_q)
+                    q_out[(n * nq + h) * D + e] = from_f32<T>(y);
+                else
+                    dst[((int64_t)(h - nq) * page_size + off) * D + e] = from_f32<T>(y);
+            }
+        __syncthreads();
+    }
+    if (!writes) return;
+    const int v0 = (nq + nkv) * dim;
+    for (int idx = threadIdx.x; idx < nkv * D; idx += blockDim.x) {
+        const int h = idx / D, e = idx - h * D;
+        const float v = e < vdim ? conv_at<T>(u, cols, taps, J, kept, n, before, v0 + h * vdim + e) : 0.f;
+        dst[(int64_t)nkv * page_size * D + ((int64_t)h * D + e) * page_size + off] = from_f32<T>(v);
+    }
+}
+
+// state row of every request of the step <- the last `kept` rows of (what it held, then the step's rows of u)
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ u, int cols, float* __restrict__ state,
+                                                          int64_t state_stride, int kept,
+                                                          const int32_t* __restrict__ cu_tokens,
+                                                          const int32_t* __restrict__ seq_slots) {
+    const int seq = blockIdx.y;
+    const int q0 = cu_tokens[seq], L = cu_tokens[seq + 1] - q0;
+    if (L <= 0) return;
+    float* row = state + (int64_t)seq_slots[seq] * state_stride;
+    for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) {
+        for (int r = 0; r < kept; ++r) {  // (r rises: a row is read before a thread of this channel overwrites it)
+            const int src = L + r;  // index into [kept old rows | L new rows]
+            row[(int64_t)r * cols + c] = src < kept ? row[(int64_t)src * cols + c]
+                                                    : to_f32<T>(u[(int64_t)(q0 + src - kept) * cols + c]);
+        }
+    }
+}
+
+extern "C" int lle_conv_norm_rope_write(const void* u, int cols, const void* taps, int J, const void* state,
+                                        int64_t state_stride, const void* token_seq, const void* cu_tokens,
+                                        const void* seq_slots, const void* slots, const void* q_weight,
+                                        const void* k_weight, const void* cos_sin, int rot, float eps, void* q_out,
+                                        void* kv_layer, int N, int nq, int nkv, int dim, int vdim, int D, int page_size,
+                                        int64_t page_stride, int write_kv, int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (J < 1 || rot % 2 || rot > dim || dim > D || vdim > D || (rot > 0 && cos_sin == nullptr) ||
+        cols < (nq + nkv) * dim + nkv * vdim)
+        return (int)hipErrorInvalidValue;
+    const size_t lds = (size_t)4 * dim * sizeof(float);
+    if (dtype == LLE_F32)
+        conv_norm_rope_write_kernel<float><<<N, 256, lds, stream>>>(
+            (const float*)u, cols, (const float*)taps, J, (const float*)state, state_stride, (const int32_t*)token_seq,
+            (const int32_t*)cu_tokens, (const int32_t*)seq_slots, (const int32_t*)slots, (const float*)q_weight,
+            (const float*)k_weight, (const float*)cos_sin, rot, eps, (float*)q_out, (float*)kv_layer, nq, nkv, dim, vdim, D,
+            page_size, page_stride, write_kv);
+    else
+        conv_norm_rope_write_kernel<bf16_t><<<N, 256, lds, stream>>>(
+            (const bf16_t*)u, cols, (const float*)taps, J, (const float*)state, state_stride, (const int32_t*)token_seq,
+            (const int32_t*)cu_tokens, (const int32_t*)seq_slots, (const int32_t*)slots, (const float*)q_weight,
+            (const float*)k_weight, (const float*)cos_sin, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, dim, vdim,
+            D, page_size, page_stride, write_kv);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int lle_conv_state_update(const void* u, int cols, void* state, int64_t state_stride, int kept,
+                                     const void* cu_tokens, const void* seq_slots, int S, int dtype,
+                                     hipStream_t stream) {
+    if (S <= 0 || kept <= 0) return 0;
+    if (S > 65535) return (int)hipErrorInvalidValue;
+    const dim3 grid((cols + 255) / 256, S);
+    if (dtype == LLE_F32)
+        conv_state_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, cols, (float*)state, state_stride, kept,
+                                                            (const int32_t*)cu_tokens, (const int32_t*)seq_slots);
+    else
+        conv_state_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, cols, (float*)state, state_stride, kept,
+                                                             (const int32_t*)cu_tokens, (const int32_t*)seq_slots);
+    LLE_RETURN_LAUNCH_STATUS();
+}
