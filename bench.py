@@ -10,6 +10,7 @@
     python bench.py --workload serving                            # requests of many lengths arriving over time
     python bench.py --workload visadra [--sizes small|mid|wide]   # Visadra beside Qwen3 at equal layer sizes, kernel by kernel
     python bench.py --workload kezasun [--sizes small|mid|wide]   # Kezasun beside Visadra, kernel by kernel
+    python bench.py --workload malilorn [--sizes small|mid|wide]  # Malilorn beside Kezasun, kernel by kernel
 
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
@@ -762,6 +763,185 @@ def kezasun_workload(args):
     print(json.dumps(line))
     return 0
 
+MALILORN_SIZES = {
+    # width, q heads, kv heads, dim, vdim, rotated, taps, wkv heads, wkv dim, decay rank, experts, top, expert ff, shared ff, dense ff
+    "small": (1024, 8, 2, 128, 128, 64, 4, 16, 64, 32, 16, 4, 512, 1024, 4096),
+    "mid": (2048, 16, 4, 128, 128, 64, 4, 32, 64, 64, 64, 6, 1408, 2816, 8192),
+    "wide": (4096, 32, 8, 128, 128, 64, 4, 64, 64, 64, 64, 6, 2048, 4096, 12288),
+}
+
+
+def malilorn_config(which, groups):
+    from litellmengine_amd.config import MalilornConfig
+
+    W, H, G, dim, vdim, rot, taps, wh, wd, rank, E, top, eff, sff, ff = MALILORN_SIZES[which]
+    mixer = {"left": {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "conv": taps,
+                      "rot": {"base": 250000.0, "dims": rot, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+             "right": {"heads": wh, "dim": wd, "decay_rank": rank}, "left_scale": 1.0, "right_scale": 0.5}
+    moe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": top}, "shared": {"ff": sff}}
+    layers = []
+    for g in range(groups):
+        layers += [{"type": "parallel", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}}] + \
+                  [{"type": "parallel", "mixer": mixer, "mlp": moe}] * 3
+    return MalilornConfig.from_dict({"architecture": "Malilorn", "vocab": 32768, "width": W, "norm": {"eps": 1e-6},
+                                     "logit_softcap": 30.0, "layers": layers})
+
+
+def malilorn_kernels(which):
+    """Each kernel of Malilorn's own at two shapes (a 2048-token prompt; 8 decoded tokens after 4096) beside the
+    like kernel of Kezasun (the closest model: the same recurrence, grouped-query attention with keys and values
+    of their own width, routed experts) at its sizes of the same name: microseconds and the share of its
+    roofline.  The recurrence's walk, its mixes and the attention itself are Kezasun's kernels and are measured
+    there (`--workload kezasun`); the attention is measured again here because it runs without a window."""
+    import torch
+
+    from litellmengine_amd.csrc.ops import default_ops
+
+    ops = default_ops()
+    W, H, G, dim, vdim, rot, taps, wh, wd, rank, E, top, eff, sff, ff = MALILORN_SIZES[which]
+    KW, kwh, kwd, krank, KH, KG, kdim, kvdim, krot, kwindow, KE, KI, ktop, keff, kng, kkeep = KEZASUN_SIZES[which]
+    dev, bf = "cuda", torch.bfloat16
+    P = PAGE_SIZE
+    rnd = lambda *shape, dtype=bf, scale=1.0: (torch.randn(shape, device=dev) * scale).to(dtype)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    out = {}
+
+    def entry(name, seconds, flops, nbytes, like=None):
+        floor = max(flops / MFMA_PEAK["bf16"], nbytes / HBM_PEAK)
+        e = {"us": round(seconds * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "frac": round(floor / seconds, 4),
+             "bound": "mfma" if flops / MFMA_PEAK["bf16"] > nbytes / HBM_PEAK else "hbm"}
+        if like is not None:
+            e["like"] = like
+            e["times_farther_from_roofline"] = round(like["frac"] / e["frac"], 2) if e["frac"] > 0 else None
+        out[name] = e
+        return e
+
+    for shape, S, q_len, past in (("prefill_2048", 1, 2048, 0), ("decode_b8_ctx4096", 8, 1, 4095)):
+        N, kv = S * q_len, past + q_len
+        pages_each = -(-kv // P)
+        table = torch.arange(S * pages_each, dtype=torch.int32, device=dev).view(S, pages_each).contiguous()
+        seq_slots, cu = ints(list(range(S))), ints([i * q_len for i in range(S + 1)])
+        kv_lens = ints([kv] * S)
+        token_seq = ints([i // q_len for i in range(N)])
+        positions = ints([past + i % q_len for i in range(N)])
+        slots = (table.long().repeat_interleave(P, 1)[:, past:kv] * P + torch.arange(past, kv, device=dev) % P).reshape(-1).int()
+        # attention over every earlier key beside Kezasun's over a window with a sink (the same kernels)
+        D = -(-max(dim, vdim) // 32) * 32
+        kv_layer = rnd(S * pages_each + 1, 2, G, P, D)
+        q = rnd(N, H, D, scale=0.1)
+        t = timed_launches(lambda: ops.paged_attention(q, kv_layer, table, seq_slots, cu, kv_lens, token_seq, None, 0.1,
+                                                       q_len, q_len, kv))
+        KD = -(-max(kdim, kvdim) // 32) * 32
+        kq, sinks = rnd(N, KH, KD, scale=0.1), torch.zeros(KH, device=dev)
+        kkv = rnd(S * pages_each + 1, 2, KG, P, KD)
+        tk = timed_launches(lambda: ops.paged_attention(kq, kkv, table, seq_slots, cu, kv_lens, token_seq, kwindow, 0.1,
+                                                        q_len, q_len, kv, sinks=sinks))
+        seen = sum(min(kwindow, past + i + 1) for i in range(q_len)) * S
+        like = entry(f"{shape}/paged_attention, window and sink (Kezasun)", tk, 4.0 * KH * KD * seen,
+                     2.0 * (S * min(kv, kwindow + q_len - 1) * 2 * KG * KD + 2 * N * KH * KD))
+        visible = S * (q_len * past + q_len * (q_len + 1) / 2)
+        entry(f"{shape}/paged_attention, every earlier key", t, 4.0 * H * D * visible,
+              2.0 * (S * kv * 2 * G * D + 2 * N * H * D), dict(like, name="paged_attention"))
+        # convolution, heads' norm, rotation and the cache write (with the state rows' update) beside the projection norm's kernel
+        cols = (H + G) * dim + G * vdim
+        u = rnd(N, cols)
+        conv_w = rnd(cols, taps, dtype=torch.float32)
+        state = torch.zeros(S + 1, (taps - 1) * cols, device=dev)
+        qw = kw = torch.ones(dim, device=dev)
+        cos_sin = ops.rope_table(positions, torch.ones(rot // 2, device=dev))
+
+        def conv():
+            ops.conv_norm_rope_write(u, conv_w, state, token_seq, cu, seq_slots, slots, qw, kw, cos_sin, rot, 1e-6, kv_layer,
+                                     H, G, dim, vdim)
+            ops.conv_state_update(u, state, taps - 1, cu, seq_slots)
+
+        t = timed_launches(conv)
+        kcols = KH * kdim + KG * (kdim + kvdim) + KH
+        kqkv, kbias = rnd(N, kcols), rnd(kcols)
+        kqw, kkw = torch.ones(KH * kdim, device=dev), torch.ones(KG * kdim, device=dev)
+        kcs = ops.rope_table(positions, torch.ones(krot // 2, device=dev))
+        tk = timed_launches(lambda: ops.proj_norm_rope_write(kqkv, kbias, slots, kqw, kkw, kcs, krot, 1e-6, kkv, KH, KG, kdim, kvdim))
+        like = entry(f"{shape}/proj_norm_rope_write (Kezasun)", tk, 0, 2.0 * N * (kcols + KH * KD + 2 * KG * KD))
+        entry(f"{shape}/conv_norm_rope_write + conv_state_update", t, 0,
+              2.0 * N * (cols + H * D + 2 * G * D) + 8.0 * S * (taps - 1) * cols, dict(like, name="proj_norm_rope_write"))
+        # the two norms around one add beside the scaled add with its norm
+        hidden, ya, yb = rnd(N, W, dtype=torch.float32), rnd(N, W), rnd(N, W, dtype=torch.float32)
+        w = torch.ones(W, device=dev)
+        t = timed_launches(lambda: ops.rmsnorm_add_rmsnorm(hidden, ya, w, 1e-6, w, 1e-6, bf, yb))
+        kh, ka, kb = rnd(N, KW, dtype=torch.float32), rnd(N, KW), rnd(N, KW, dtype=torch.float32)
+        kwn = torch.ones(KW, device=dev)
+        tk = timed_launches(lambda: ops.scaled_add_rmsnorm(kh, ka, kb, 0.3, kwn, 1e-6, bf))
+        like = entry(f"{shape}/scaled_add_rmsnorm (Kezasun)", tk, 0, N * KW * (4 + 4 + 2 + 4 + 2.0))
+        entry(f"{shape}/rmsnorm_add_rmsnorm", t, 0, N * W * (4 + 4 + 2 + 4 + 2.0), dict(like, name="scaled_add_rmsnorm"))
+        # activations: gated relu with biases (dense), squared relu with a row gate (shared expert) beside silu_mul
+        z2, b2 = rnd(N, 2 * ff), rnd(2 * ff)
+        t = timed_launches(lambda: ops.bias_act(z2, "relu", True, bias=b2))
+        ts = timed_launches(lambda: ops.silu_mul(z2))
+        like = entry(f"{shape}/silu_mul (Qwen3)", ts, 0, 2.0 * N * 3 * ff)
+        entry(f"{shape}/bias_act, gated relu with biases", t, 0, 2.0 * N * 3 * ff, dict(like, name="silu_mul"))
+        # the routers and the experts
+        logits = rnd(N, E + 1, dtype=torch.float32)
+        t = timed_launches(lambda: ops.moe_route(logits, None, top, score="sigmoid", experts=E))
+        klogits, kcorr = rnd(N, KE + KI, dtype=torch.float32), torch.zeros(KE + KI, device=dev)
+        tk = timed_launches(lambda: ops.moe_route_grouped(klogits, kcorr, ktop, kng, kkeep))
+        like = entry(f"{shape}/moe_route_grouped (Kezasun)", tk, 0, N * (4.0 * (KE + KI) + 8 * ktop))
+        entry(f"{shape}/moe_route, sigmoid scores", t, 0, N * (4.0 * (E + 1) + 8 * top), dict(like, name="moe_route_grouped"))
+        xx = rnd(N, W, scale=0.1)
+        up, down = rnd(E, eff, W, scale=0.02), rnd(E, W, eff, scale=0.02)
+        ids, gains = ops.moe_route(logits, None, top, score="sigmoid", experts=E)
+        t = timed_launches(lambda: ops.moe_experts(xx, ids, gains, up, down, form="relu2", gain_on_input=True), repeats=5)
+        kx = rnd(N, KW, scale=0.1)
+        kgu, kdown = rnd(KE, 2 * keff, KW, scale=0.02), rnd(KE, KW, keff, scale=0.02)
+        kids, kgains = ops.moe_route_grouped(klogits, kcorr, ktop, kng, kkeep)
+        tk = timed_launches(lambda: ops.moe_experts(kx, kids, kgains, kgu, kdown), repeats=5)
+        real = int((kids < KE).sum())
+        like = entry(f"{shape}/moe_experts with identity experts (Kezasun)", tk, 6.0 * real * KW * keff,
+                     2.0 * (3 * min(KE, real) * KW * keff + 2 * N * KW))
+        entry(f"{shape}/moe_experts, no gate, weighted at the input", t, 4.0 * N * top * W * eff,
+              2.0 * (2 * min(E, N * top) * W * eff + 2 * N * W), dict(like, name="moe_experts"))
+        # the cap on the logits beside the scaling of the logits (the wanted rows: one a request)
+        lg = rnd(S, 32768, dtype=torch.float32)
+        t = timed_launches(lambda: ops.softcap_(lg, 30.0))
+        tk = timed_launches(lambda: ops.scale_(lg, 1.0))
+        like = entry(f"{shape}/scale_ (Visadra)", tk, 0, 8.0 * S * 32768)
+        entry(f"{shape}/softcap_", t, 0, 8.0 * S * 32768, dict(like, name="scale_"))
+        del kv_layer, kkv
+    return out
+
+
+def malilorn_workload(args):
+    import torch
+
+    from litellmengine_amd.models import random_model
+
+    which = args.sizes if args.sizes in MALILORN_SIZES else "mid"
+    groups = max(1, args.layers // 4) if args.layers != SIZES["num_hidden_layers"] else 1
+    mcfg = malilorn_config(which, groups)
+    kcfg = kezasun_config(which, 2 * groups)
+    line = {"metric": f"Malilorn beside Kezasun at layer sizes of the same name ({which}): prefill tok/s @ 2048 and decode tok/s "
+                      f"@ batch {args.batch}, context {args.context}", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic: seeded random weights, uniform random token ids", "higher_is_better": True,
+            "config": {"sizes": dict(zip(("width", "heads", "kv_heads", "dim", "vdim", "rotated", "taps", "wkv_heads", "wkv_dim",
+                                          "decay_rank", "experts", "top", "expert_ff", "shared_ff", "dense_ff"),
+                                         MALILORN_SIZES[which])),
+                       "layers": 4 * groups,
+                       "pattern": "every layer attention behind a convolution beside a recurrence; dense, moe, moe, moe",
+                       "beside": f"Kezasun with {8 * groups} layers: as many attentions and as many recurrences, twice the feed-forwards"}}
+    steps, warmup = min(args.steps, 16), min(args.warmup, 4)
+    for name, cfg in (("malilorn", mcfg), ("kezasun", kcfg)):
+        model = random_model(cfg, seed=0, dtype="bfloat16")
+        dt = time_decode(model, cfg, args.batch, args.context, steps, warmup)
+        pt = time_prefill(model, cfg, PREFILL_TOKENS)
+        line[name] = {"decode_tok_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                      "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
+        del model
+        torch.cuda.empty_cache()
+    line["value"] = line["malilorn"]["decode_tok_s"]
+    line["steps"], line["warmup"] = steps, warmup
+    line["kernels"] = malilorn_kernels(which)
+    print(json.dumps(line))
+    return 0
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -776,12 +956,12 @@ def main():
     ap.add_argument("--no-more", action="store_true", help="skip the other workloads that the default line carries")
     ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b", "small", "mid", "wide"],
                     help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B; "
-                         "small, mid or wide: the layer sizes of --workload visadra and --workload kezasun")
-    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra", "kezasun"],
+                         "small, mid or wide: the layer sizes of --workload visadra, kezasun and malilorn")
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra", "kezasun", "malilorn"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
                          "sizes, a mixed prompt-portion + decode step at Qwen3-32B sizes, requests arriving over time, "
-                         "Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline, or Kezasun "
-                         "beside Visadra the same way")
+                         "Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline, Kezasun "
+                         "beside Visadra the same way, or Malilorn beside Kezasun the same way")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
@@ -799,6 +979,8 @@ def main():
             return visadra_workload(args)
         if args.workload == "kezasun":
             return kezasun_workload(args)
+        if args.workload == "malilorn":
+            return malilorn_workload(args)
         args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
         return mixed_workload(args)
 

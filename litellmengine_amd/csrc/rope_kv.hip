@@ -600,6 +600,176 @@ __global__ __launch_bounds__(256) void conv_norm_rope_write_kernel(
     }
 }
 
+// The same for up to CV_MAX_TAPS taps and heads of up to 64 CV_ITEMS elements, which is what models have: a
+// wavefront per (head, run of `tile` consecutive tokens), grid (token tiles, heads / 4); the v part of a row
+// counts as heads of its own (no norm, no rotation).  A lane owns up to CV_ITEMS items of its head, an item being
+// a rotated pair (element i and i + rot / 2) or one element past the rotation: the partner of a rotation sits in
+// the same lane, the norm's sum crosses the lanes once, nothing passes through LDS and no barrier is met.  The
+// lane keeps its channels' taps and the last J - 1 values of u in registers and walks its tokens in order: while
+// the request stays the same a token costs one new load per channel, whatever J.
+#define CV_MAX_TAPS 8
+#define CV_ITEMS 4
+
+template <typename T, int J>
+__global__ __launch_bounds__(256) void conv_norm_rope_write_tile_kernel(
+    const T* __restrict__ u, int cols, const float* __restrict__ taps, const float* __restrict__ state,
+    int64_t state_stride, const int32_t* __restrict__ token_seq, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ slots, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, const float* __restrict__ cos_sin, int rot, float eps, T* __restrict__ q_out,
+    T* __restrict__ kv_layer, int N, int nq, int nkv, int dim, int vdim, int D, int page_size, int64_t page_stride,
+    int write_kv, int tile) {
+    constexpr int W = J > 1 ? J - 1 : 1;
+    const int lane = threadIdx.x % LLE_WAVE;
+    const int h = blockIdx.y * (blockDim.x / LLE_WAVE) + threadIdx.x / LLE_WAVE;
+    if (h >= nq + (write_kv ? 2 * nkv : 0)) return;  // (the whole wavefront; no barrier follows)
+    const bool is_q = h < nq, is_v = h >= nq + nkv;
+    const int width = is_v ? vdim : dim;
+    const int hrot = is_v ? 0 : rot, half = hrot / 2;
+    const int items = half + (width - hrot);
+    const int col0 = is_q ? h * dim : is_v ? (nq + nkv) * dim + (h - nq - nkv) * vdim : nq * dim + (h - nq) * dim;
+    const float* nw = is_q ? q_weight : k_weight;
+    int ca[CV_ITEMS], cb[CV_ITEMS];  // the item's elements of the head (cb < 0: no partner)
+    float ta[CV_ITEMS][J], tb[CV_ITEMS][J], wa[CV_ITEMS], wb[CV_ITEMS], xa[CV_ITEMS][W], xb[CV_ITEMS][W];
+#pragma unroll
+    for (int i = 0; i < CV_ITEMS; ++i) {
+        const int it = lane + LLE_WAVE * i;
+        ca[i] = it < half ? it : hrot + (it - half);
+        cb[i] = it < half ? it + half : -1;
+        if (it >= items) ca[i] = -1;
+        wa[i] = wb[i] = 1.f;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            ta[i][j] = ca[i] >= 0 ? taps[(int64_t)(col0 + ca[i]) * J + j] : 0.f;
+            tb[i][j] = (ca[i] >= 0 && cb[i] >= 0) ? taps[(int64_t)(col0 + cb[i]) * J + j] : 0.f;
+        }
+        if (!is_v && ca[i] >= 0) {
+            wa[i] = nw[ca[i]];
+            if (cb[i] >= 0) wb[i] = nw[cb[i]];
+        }
+#pragma unroll
+        for (int j = 0; j < W; ++j) xa[i][j] = xb[i][j] = 0.f;
+    }
+    const int64_t n0 = (int64_t)blockIdx.x * tile;
+    int prev_seq = -1;
+    for (int tk = 0; tk < tile; ++tk) {
+        const int64_t n = n0 + tk;
+        if (n >= N) break;
+        const int seq = token_seq[n];
+        float va[CV_ITEMS], vb[CV_ITEMS];
+        if (seq != prev_seq && J > 1) {  // the first token of this wavefront's run, or another request: fill the window
+            const int before = (int)(n - cu_tokens[seq]);
+            const float* kept = state ? state + (int64_t)seq_slots[seq] * state_stride : nullptr;
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                const int back = J - 1 - j;
+#pragma unroll
+                for (int i = 0; i < CV_ITEMS; ++i) {
+                    float a = 0.f, b = 0.f;
+                    if (ca[i] >= 0) {
+                        if (back <= before) {
+                            a = to_f32<T>(u[(n - back) * cols + col0 + ca[i]]);
+                            if (cb[i] >= 0) b = to_f32<T>(u[(n - back) * cols + col0 + cb[i]]);
+                        } else if (kept) {
+                            const int64_t r = (int64_t)(J - 1 - (back - before)) * cols + col0;
+                            a = kept[r + ca[i]];
+                            if (cb[i] >= 0) b = kept[r + cb[i]];
+                        }
+                    }
+                    xa[i][j] = a;
+                    xb[i][j] = b;
+                }
+            }
+        }
+        prev_seq = seq;
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < CV_ITEMS; ++i) {
+            float a = 0.f, b = 0.f;
+            if (ca[i] >= 0) {
+                a = to_f32<T>(u[n * cols + col0 + ca[i]]);
+                if (cb[i] >= 0) b = to_f32<T>(u[n * cols + col0 + cb[i]]);
+            }
+            float sa = ta[i][J - 1] * a, sb = tb[i][J - 1] * b;
+#pragma unroll
+            for (int j = 0; j < J - 1; ++j) {
+                sa += ta[i][j] * xa[i][j];
+                sb += tb[i][j] * xb[i][j];
+            }
+#pragma unroll
+            for (int j = 0; j + 1 < J - 1; ++j) {  // the window moves on by one token
+                xa[i][j] = xa[i][j + 1];
+                xb[i][j] = xb[i][j + 1];
+            }
+            if (J > 1) {
+                xa[i][W - 1] = a;
+                xb[i][W - 1] = b;
+            }
+            va[i] = sa;
+            vb[i] = sb;
+            ss += sa * sa + sb * sb;
+        }
+        const int slot = slots[n];
+        const bool writes = is_q || slot >= 0;
+        const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - page * page_size : 0;
+        T* dst = kv_layer + (int64_t)page * page_stride;
+        if (is_v) {
+            if (!writes) continue;
+            T* vt = dst + (int64_t)nkv * page_size * D + (int64_t)(h - nq - nkv) * D * page_size + off;
+#pragma unroll
+            for (int i = 0; i < CV_ITEMS; ++i)
+                if (ca[i] >= 0) vt[(int64_t)ca[i] * page_size] = from_f32<T>(va[i]);
+            for (int e = vdim + lane; e < D; e += LLE_WAVE) vt[(int64_t)e * page_size] = from_f32<T>(0.f);
+            continue;
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+        if (!writes) continue;
+        T* row = is_q ? q_out + (n * nq + h) * D : dst + ((int64_t)(h - nq) * page_size + off) * D;
+        const float* cs = cos_sin + n * rot;  // [rot / 2][2]
+#pragma unroll
+        for (int i = 0; i < CV_ITEMS; ++i) {
+            if (ca[i] < 0) continue;
+            const float a = va[i] * inv * wa[i];
+            if (cb[i] >= 0) {
+                const float b = vb[i] * inv * wb[i];
+                const float c = cs[2 * ca[i]], sn = cs[2 * ca[i] + 1];
+                row[ca[i]] = from_f32<T>(a * c - b * sn);
+                row[cb[i]] = from_f32<T>(b * c + a * sn);
+            } else {
+                row[ca[i]] = from_f32<T>(a);
+            }
+        }
+        for (int e = dim + lane; e < D; e += LLE_WAVE) row[e] = from_f32<T>(0.f);
+    }
+}
+
+template <typename T>
+static bool conv_tile_launch(int J, dim3 grid, hipStream_t stream, const void* u, int cols, const void* taps,
+                             const void* state, int64_t state_stride, const void* token_seq, const void* cu_tokens,
+                             const void* seq_slots, const void* slots, const void* q_weight, const void* k_weight,
+                             const void* cos_sin, int rot, float eps, void* q_out, void* kv_layer, int N, int nq, int nkv,
+                             int dim, int vdim, int D, int page_size, int64_t page_stride, int write_kv, int tile) {
+#define LLE_CONV_CASE(JJ)                                                                                               \
+    case JJ:                                                                                                            \
+        conv_norm_rope_write_tile_kernel<T, JJ><<<grid, 256, 0, stream>>>(                                              \
+            (const T*)u, cols, (const float*)taps, (const float*)state, state_stride, (const int32_t*)token_seq,        \
+            (const int32_t*)cu_tokens, (const int32_t*)seq_slots, (const int32_t*)slots, (const float*)q_weight,        \
+            (const float*)k_weight, (const float*)cos_sin, rot, eps, (T*)q_out, (T*)kv_layer, N, nq, nkv, dim, vdim, D, \
+            page_size, page_stride, write_kv, tile);                                                                    \
+        return true;
+    switch (J) {
+        LLE_CONV_CASE(1)
+        LLE_CONV_CASE(2)
+        LLE_CONV_CASE(3)
+        LLE_CONV_CASE(4)
+        LLE_CONV_CASE(5)
+        LLE_CONV_CASE(6)
+        LLE_CONV_CASE(7)
+        LLE_CONV_CASE(8)
+    }
+#undef LLE_CONV_CASE
+    return false;
+}
+
 // state row of every request of the step <- the last `kept` rows of (what it held, then the step's rows of u)
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_kernel(const T* __restrict__ u, int cols, float* __restrict__ state,
@@ -629,6 +799,25 @@ extern "C" int lle_conv_norm_rope_write(const void* u, int cols, const void* tap
     if (J < 1 || rot % 2 || rot > dim || dim > D || vdim > D || (rot > 0 && cos_sin == nullptr) ||
         cols < (nq + nkv) * dim + nkv * vdim)
         return (int)hipErrorInvalidValue;
+    if (J <= CV_MAX_TAPS && dim <= CV_ITEMS * LLE_WAVE && vdim <= CV_ITEMS * LLE_WAVE) {
+        // runs of tokens long enough that the taps are loaded seldom, short enough that a prompt fills the chip
+        // (measured at 2048 tokens: runs of 16 tokens where that leaves some 768 workgroups, shorter runs otherwise)
+        const int heads = nq + (write_kv ? 2 * nkv : 0);
+        const int64_t fit = (int64_t)N * ((heads + 3) / 4) / 768;
+        const int tile = fit >= 16 ? 16 : fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : 1;
+        const dim3 grid((N + tile - 1) / tile, (heads + 3) / 4);
+        if (grid.y <= 65535) {
+            if (dtype == LLE_F32)
+                conv_tile_launch<float>(J, grid, stream, u, cols, taps, state, state_stride, token_seq, cu_tokens, seq_slots,
+                                        slots, q_weight, k_weight, cos_sin, rot, eps, q_out, kv_layer, N, nq, nkv, dim, vdim,
+                                        D, page_size, page_stride, write_kv, tile);
+            else
+                conv_tile_launch<bf16_t>(J, grid, stream, u, cols, taps, state, state_stride, token_seq, cu_tokens,
+                                         seq_slots, slots, q_weight, k_weight, cos_sin, rot, eps, q_out, kv_layer, N, nq, nkv,
+                                         dim, vdim, D, page_size, page_stride, write_kv, tile);
+            LLE_RETURN_LAUNCH_STATUS();
+        }
+    }
     const size_t lds = (size_t)4 * dim * sizeof(float);
     if (dtype == LLE_F32)
         conv_norm_rope_write_kernel<float><<<N, 256, lds, stream>>>(

@@ -47,11 +47,12 @@ def batch(q_lens):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("sizes", [  # nq, nkv, dim, vdim, D, rot, taps, page size
     (6, 2, 24, 40, 64, 8, 3, 4), (8, 1, 128, 96, 128, 64, 4, 16), (1, 1, 48, 10, 64, 2, 1, 8), (5, 5, 8, 12, 32, 0, 5, 16),
-    (4, 2, 64, 64, 64, 64, 2, 16)])
+    (4, 2, 64, 64, 64, 64, 2, 16), (2, 1, 16, 24, 32, 4, 9, 8), (3, 1, 256, 200, 256, 100, 8, 16)])
 @pytest.mark.parametrize("q_lens", [[1, 1, 1], [7, 1, 2, 30], [70]])
 def test_conv_norm_rope_write_and_its_state(dtype, sizes, q_lens):
     """Single tokens, portions shorter and longer than the taps reach, from state rows that are not zero and are
-    columns of a wider row; a padding row (page slot -1) writes nothing; the state is advanced afterwards."""
+    columns of a wider row; a padding row (page slot -1) writes nothing; the state is advanced afterwards.  Up to
+    eight taps take the kernel that walks runs of tokens with the window in registers, nine the plain one."""
     o = ops()
     nq, nkv, dim, vdim, D, rot, J, P = sizes
     seq_slots, cu, token_seq, N = batch(q_lens)
