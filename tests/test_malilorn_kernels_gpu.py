@@ -88,6 +88,37 @@ def test_conv_norm_rope_write_and_its_state(dtype, sizes, q_lens):
             assert torch.equal(state[int(seq_slots[s]), (J - 2) * cols :], last)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_lens,heads", [([1, 300, 2, 700, 1, 1, 45], (8, 2)), ([3, 1500, 1, 2, 1400, 5, 90, 1], (12, 4)),
+                                          ([5000], (4, 4))])
+def test_conv_runs_of_tokens_across_requests(dtype, q_lens, heads):
+    """Steps long enough that a wavefront walks runs of 4, 8 and 16 tokens with its window in registers: requests
+    begin and end inside the runs, single tokens sit between long portions, the states are not zero."""
+    o = ops()
+    (nq, nkv), dim, vdim, D, rot, J, P = heads, 32, 48, 64, 16, 4, 16
+    seq_slots, cu, token_seq, N = batch(q_lens)
+    cols = (nq + nkv) * dim + nkv * vdim
+    u = rnd((N, cols), dtype, 1)
+    taps = rnd((cols, J), torch.float32, 2, 0.5)
+    state = rnd((9, (J - 1) * cols), torch.float32, 3)
+    qw, kw = 1.0 + rnd((dim,), torch.float32, 4, 0.2), 1.0 + rnd((dim,), torch.float32, 5, 0.2)
+    angles = rnd((N, rot // 2), torch.float32, 6, 3.0)
+    cos_sin = torch.stack([torch.cos(angles), torch.sin(angles)], dim=-1).contiguous()
+    pages = -(-N // P) + 1
+    slots = torch.randperm(pages * P, generator=torch.Generator().manual_seed(7))[:N].to(torch.int32).cuda()
+    kv = torch.zeros((pages, 2, nkv, P, D), dtype=dtype).cuda()
+    want_kv, want_state = kv.clone(), state.clone()
+    want = REF.conv_norm_rope_write(u, taps, want_state, token_seq, cu, seq_slots, slots, qw, kw, cos_sin, rot, 1e-5, want_kv,
+                                    nq, nkv, dim, vdim)
+    got = o.conv_norm_rope_write(u, taps, state, token_seq, cu, seq_slots, slots, qw, kw, cos_sin, rot, 1e-5, kv, nq, nkv, dim,
+                                 vdim)
+    assert (got.double() - want.double()).abs().max() < tol(dtype, 8)
+    assert (kv.double() - want_kv.double()).abs().max() < tol(dtype, 8)
+    REF.conv_state_update(u, want_state, J - 1, cu, seq_slots)
+    o.conv_state_update(u, state, J - 1, cu, seq_slots)
+    assert torch.equal(state, want_state)
+
+
 def test_conv_portions_equal_one_go():
     """A request's tokens in one step, and the same tokens in steps of 1, 2, 3, 1, ... through the state rows."""
     o = ops()
@@ -114,9 +145,11 @@ def test_conv_portions_equal_one_go():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["silu", "relu", "relu2"])
 @pytest.mark.parametrize("gated", [False, True])
-def test_bias_act(dtype, kind, gated):
+@pytest.mark.parametrize("F", [52, 72])
+def test_bias_act(dtype, kind, gated, F):
+    """Rows of a multiple of 8 take 16-byte pieces in bfloat16, others one element a thread."""
     o = ops()
-    N, F = 37, 52
+    N = 37
     z = rnd((N, 2 * F if gated else F), dtype, 1, 2.0)
     bias = rnd((z.shape[1],), dtype, 2)
     gate = rnd((N, 7), torch.float32, 3, 2.0)
