@@ -220,6 +220,27 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, layers_out: Optional[
     return cap * torch.tanh(logits / cap) if cap else logits
 
 
+def router_margins(cfg: dict, w: Dict[str, torch.Tensor], tokens) -> torch.Tensor:
+    """[T]: per position the smallest gap, over the routed layers, between the last chosen expert's logit and the
+    best one left out (infinity where nothing is left out): where it is tiny, rounding decides the choice."""
+    eps = cfg["norm"]["eps"]
+    x = w["embed"][torch.as_tensor(list(tokens), dtype=torch.long)]
+    gap = torch.full((x.shape[0],), float("inf"), dtype=x.dtype)
+    for i, spec in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        x = x + rms_norm(parallel_mixer(rms_norm(x, w[p + "norm1"], eps), w, p + "mix.", spec["mixer"], eps), w[p + "norm1b"], eps)
+        f = spec.get("mlp")
+        if not f:
+            continue
+        h = rms_norm(x, w[p + "norm2"], eps)
+        if f.get("kind") != "dense" and f["router"]["experts"] > f["router"]["top"]:
+            z = torch.sort(h @ w[p + "mlp.router"].T, dim=-1, descending=True).values
+            top = f["router"]["top"]
+            gap = torch.minimum(gap, z[:, top - 1] - z[:, top])
+        x = x + rms_norm(feed_forward(h, w, p + "mlp.", f), w[p + "norm2b"], eps)
+    return gap
+
+
 def load(model_dir: str, dtype=torch.float64):
     from safetensors.torch import load_file
 
