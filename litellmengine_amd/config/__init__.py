@@ -2,6 +2,7 @@ from .model_config import ConfigError, Qwen3Config, read_config_json, FULL_ATTEN
 from .visadra_config import VisadraConfig
 from .kezasun_config import KezasunConfig
 from .malilorn_config import MalilornConfig
+from .birelix_config import BirelixConfig
 from .registry import (
     Architecture,
     architecture_of,
@@ -18,6 +19,7 @@ __all__ = [
     "VisadraConfig",
     "KezasunConfig",
     "MalilornConfig",
+    "BirelixConfig",
     "FULL_ATTENTION",
     "SLIDING_ATTENTION",
     "architecture_of",

@@ -36,6 +36,7 @@ LIBRARIES: Dict[str, List[str]] = {
     "latent": ["latent.hip"],
     "moe": ["moe.hip"],
     "wkv": ["wkv.hip"],
+    "delta": ["delta.hip"],
     "probe": ["probe.hip"],
 }
 # libraries without GPU code: compiled with the host's C++ compiler

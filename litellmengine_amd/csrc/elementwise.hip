@@ -225,14 +225,17 @@ extern "C" int lle_tanh(void* x, int64_t total, int dtype, hipStream_t stream) {
 //   gated:  out[n, f] = act(z[n, f] + b[f]) * (z[n, F + f] + b[F + f])        z [N, 2 F]
 //   plain:  out[n, f] = act(z[n, f] + b[f])                                   z [N, F]
 // times sigmoid(row_gate[n * gate_stride + gate_col]) where a row gate is given (float32).
-// act: 0 silu, 1 relu, 2 the square of relu.  `b` may be null.  Everything in 32-bit.
+// act: 0 silu, 1 relu, 2 the square of relu, 3 gelu in its tanh form.  `b` may be null.  Everything in 32-bit.
 // ---------------------------------------------------------------------------------
 #define LLE_ACT_SILU 0
 #define LLE_ACT_RELU 1
 #define LLE_ACT_RELU2 2
+#define LLE_ACT_GELU_TANH 3
 
 __device__ __forceinline__ float apply_act(float x, int kind) {
     if (kind == LLE_ACT_SILU) return x / (1.0f + expf(-x));
+    if (kind == LLE_ACT_GELU_TANH)  // 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+        return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
     const float r = fmaxf(x, 0.f);
     return kind == LLE_ACT_RELU ? r : r * r;
 }
@@ -296,6 +299,7 @@ static void bias_act_vec(const void* z, const void* bias, const void* row_gate, 
                                                                     (bf16_t*)out, total8, F8)
     if (kind == LLE_ACT_SILU) LLE_ACT_CASE(LLE_ACT_SILU);
     else if (kind == LLE_ACT_RELU) LLE_ACT_CASE(LLE_ACT_RELU);
+    else if (kind == LLE_ACT_GELU_TANH) LLE_ACT_CASE(LLE_ACT_GELU_TANH);
     else LLE_ACT_CASE(LLE_ACT_RELU2);
 #undef LLE_ACT_CASE
 }
@@ -303,7 +307,7 @@ static void bias_act_vec(const void* z, const void* bias, const void* row_gate, 
 extern "C" int lle_bias_act(const void* z, const void* bias, const void* row_gate, int gate_stride, int gate_col,
                             void* out, int N, int F, int gated, int kind, int dtype, hipStream_t stream) {
     if (N <= 0 || F <= 0) return 0;
-    if (kind < 0 || kind > LLE_ACT_RELU2) return (int)hipErrorInvalidValue;
+    if (kind < 0 || kind > LLE_ACT_GELU_TANH) return (int)hipErrorInvalidValue;
     if (dtype == LLE_BF16 && F % 8 == 0) {
         if (gated) bias_act_vec<1>(z, bias, row_gate, gate_stride, gate_col, out, (int64_t)N * F / 8, F / 8, kind, stream);
         else bias_act_vec<0>(z, bias, row_gate, gate_stride, gate_col, out, (int64_t)N * F / 8, F / 8, kind, stream);

@@ -149,7 +149,9 @@ __global__ __launch_bounds__(LAT_TILE) void latent_attention_generic_kernel(
     for (int i = tid; i < rot; i += LAT_TILE) qr[i] = qrs[i];
     __syncthreads();
 
-    float m = sink[h], l = 1.0f;  // the sink: a key with score `sink` and no value
+    // the sink: a key with score `sink` and no value; without one the sum starts empty (the first tile holds
+    // the token itself, so the maximum is finite from there on)
+    float m = sink ? sink[h] : -INFINITY, l = sink ? 1.0f : 0.0f;
     float acc[LAT_MAX_RANK_PER_THREAD];
 #pragma unroll
     for (int k = 0; k < LAT_MAX_RANK_PER_THREAD; ++k) acc[k] = 0.f;
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     for (int u = 0; u < RT; ++u) {
 #pragma unroll
         for (int i = 0; i < NT; ++i) o[u][i] = lf32x4{0.f, 0.f, 0.f, 0.f};
-        const bool first = split == 0 && valid[u];
+        const bool first = split == 0 && valid[u] && sink != nullptr;
         m[u] = first ? sink[head[u]] * LAT_LOG2E : LAT_NEG_BIG;     // base 2; the same in the row's lanes of every wavefront
         l[u] = (first && c == 0 && wave == 0) ? 1.0f : 0.0f;        // this lane's share of the row's sum
     }

@@ -8,6 +8,9 @@ MAX_HEAD_DIM = 256  # the attention kernels keep a head's elements in four regis
 MAX_SUMMED_NORM_WIDTH = 8192
 # the recurrence with a matrix state keeps a head's key channels in registers, a quarter per thread
 MAX_WKV_HEAD_DIM = 256
+# the delta rule's walk keeps a column of a head's state in the registers of sixteen lanes, up to sixteen each;
+# its convolution keeps a head in a wavefront, four elements a lane
+MAX_DELTA_HEAD_DIM = 256
 
 
 def check_head_dim(head_dim: int, rotary_dim: int = 0) -> None:

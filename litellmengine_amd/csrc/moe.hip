@@ -88,15 +88,17 @@ extern "C" int lle_moe_route(const void* logits, const void* bias, void* ids, vo
 }
 
 
-// A router whose scores are the softmax over ALL experts and whose choice is limited to groups: one wavefront per
-// token.  scores s = softmax(logits); choice scores c = s + correction; the experts form `groups` equal groups of
-// neighbours, a group's score is its largest c, and only the `keep` best groups' experts can be chosen (the lower
-// index wins a tie, among groups and among experts); gains = s of the chosen / (their sum + 1e-20).
+// A router whose choice is limited to groups: one wavefront per token.  Scores s = softmax(logits) over ALL experts
+// (`sigmoid`: the sigmoid of every logit on its own); choice scores c = s + correction (none: c = s); the experts
+// form `groups` equal groups of neighbours, a group's score is the sum of its `group_top` largest c (1: its
+// largest), and only the `keep` best groups' experts can be chosen (the lower index wins a tie, among groups and
+// among experts); gains = s of the chosen / (their sum + 1e-20).
 // Dynamic LDS: per wavefront E scores, E choice scores and `groups` group scores.
 __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __restrict__ logits,
                                                                  const float* __restrict__ correction,
                                                                  int32_t* __restrict__ ids, float* __restrict__ gains,
-                                                                 int N, int E, int top, int groups, int keep) {
+                                                                 int N, int E, int top, int groups, int keep, int sigmoid,
+                                                                 int group_top) {
     extern __shared__ float route_smem[];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int n = min(blockIdx.x * (blockDim.x / LLE_WAVE) + wave, N - 1);  // (a wavefront past the end repeats the last token)
@@ -104,27 +106,53 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __r
     float* c = s + E;
     float* best = c + E;
     const float* row = logits + (int64_t)n * E;
-    float big = -INFINITY;
-    for (int e = lane; e < E; e += LLE_WAVE) big = fmaxf(big, row[e]);
-    big = wave_max(big);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += LLE_WAVE) {
-        const float x = expf(row[e] - big);
-        s[e] = x;
-        sum += x;
-    }
-    sum = wave_sum(sum);
-    for (int e = lane; e < E; e += LLE_WAVE) {
-        const float x = s[e] / sum;
-        s[e] = x;
-        c[e] = x + correction[e];
+    if (sigmoid) {
+        for (int e = lane; e < E; e += LLE_WAVE) {
+            const float x = 1.0f / (1.0f + expf(-row[e]));
+            s[e] = x;
+            c[e] = x + (correction ? correction[e] : 0.f);
+        }
+    } else {
+        float big = -INFINITY;
+        for (int e = lane; e < E; e += LLE_WAVE) big = fmaxf(big, row[e]);
+        big = wave_max(big);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += LLE_WAVE) {
+            const float x = expf(row[e] - big);
+            s[e] = x;
+            sum += x;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += LLE_WAVE) {
+            const float x = s[e] / sum;
+            s[e] = x;
+            c[e] = x + (correction ? correction[e] : 0.f);
+        }
     }
     __syncthreads();
     const int size = E / groups;
     for (int g = lane; g < groups; g += LLE_WAVE) {
-        float b = c[g * size];
-        for (int i = 1; i < size; ++i) b = fmaxf(b, c[g * size + i]);
-        best[g] = b;
+        // the group's largest choice scores, one after the other: each the best of those that come behind
+        // the one before it in the order (larger first, among equals the lower index first)
+        float worth = 0.f, pv = INFINITY;
+        int pi = -1;
+        for (int t = 0; t < min(group_top, size); ++t) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int i = 0; i < size; ++i) {
+                const float v = c[g * size + i];
+                const bool behind = v < pv || (v == pv && i > pi);
+                if (behind && (bi < 0 || v > bv)) {
+                    bv = v;
+                    bi = i;
+                }
+            }
+            if (bi < 0) break;
+            worth = t == 0 ? bv : worth + bv;
+            pv = bv;
+            pi = bi;
+        }
+        best[g] = worth;
     }
     __syncthreads();
     if (keep < groups) {
@@ -170,15 +198,16 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __r
 }
 
 extern "C" int lle_moe_route_grouped(const void* logits, const void* correction, void* ids, void* gains, int N, int E,
-                                     int top, int groups, int keep, hipStream_t stream) {
+                                     int top, int groups, int keep, int sigmoid, int group_top, hipStream_t stream) {
     if (N <= 0) return 0;
     if (top <= 0 || top > MOE_MAX_TOP || top > E || groups <= 0 || E % groups || keep <= 0 || keep > groups ||
-        top > keep * (E / groups))
+        top > keep * (E / groups) || group_top < 1)
         return (int)hipErrorInvalidValue;
     const size_t lds = (size_t)4 * (2 * E + groups) * sizeof(float);
     if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
     moe_route_grouped_kernel<<<(N + 3) / 4, 256, lds, stream>>>((const float*)logits, (const float*)correction,
-                                                                   (int32_t*)ids, (float*)gains, N, E, top, groups, keep);
+                                                                   (int32_t*)ids, (float*)gains, N, E, top, groups, keep,
+                                                                   sigmoid, group_top);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -210,8 +239,21 @@ __device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __re
 // MOE_PLAIN_RELU2: act = relu(Wu x)^2, weights [E, F, K].  `in_gains` (or null): the pair's gain multiplies the
 // expert's INPUT, which is a factor on its first products' results; it is applied there, in 32-bit, before the
 // activation (the gain then takes no part in the sum of the experts' results).
+// MOE_GATED_CLAMP: the gated layout with g = min(Wg x, limit), u = clamp(Wu x, -limit, limit),
+// act = g sigmoid(1.702 g) (u + 1).
 #define MOE_GATED_SILU 0
 #define MOE_PLAIN_RELU2 1
+#define MOE_GATED_CLAMP 2
+
+template <int FORM>
+__device__ __forceinline__ float moe_gated_act(float g, float u, float limit) {
+    if (FORM == MOE_GATED_CLAMP) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
 
 __device__ __forceinline__ float moe_relu2(float z) {
     const float r = fmaxf(z, 0.f);
@@ -223,7 +265,7 @@ template <typename T, int FORM>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids,
                                                            const T* __restrict__ gate_up,
                                                            const float* __restrict__ in_gains, T* __restrict__ act,
-                                                           int top, int F, int K, int E) {
+                                                           int top, int F, int K, int E, float limit) {
     const int p = blockIdx.x;
     const int f = blockIdx.y * 4 + threadIdx.x / LLE_WAVE;
     if (f >= F) return;
@@ -240,7 +282,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
     const T* w = gate_up + (int64_t)e * 2 * F * K;
     const float g = gain * wave_dot<T>(xr, w + (int64_t)f * K, K);
     const float u = gain * wave_dot<T>(xr, w + (int64_t)(F + f) * K, K);
-    if (threadIdx.x % LLE_WAVE == 0) act[(int64_t)p * F + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    if (threadIdx.x % LLE_WAVE == 0) act[(int64_t)p * F + f] = from_f32<T>(moe_gated_act<FORM>(g, u, limit));
 }
 
 // grid (tokens, ceil(H / 4)), 4 wavefronts: wavefront w makes out[n, o], o = 4 blockIdx.y + w
@@ -270,16 +312,19 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
 template <typename T>
 static void moe_experts_pairs(const void* x, const void* ids, const void* gains, const void* gate_up, const void* down,
                               void* act, void* out, int N, int top, int E, int F, int K, int H, int form,
-                              int gain_on_input, hipStream_t stream) {
+                              int gain_on_input, float limit, hipStream_t stream) {
     const dim3 g1(N * top, (F + 3) / 4), g2(N, (H + 3) / 4);
     const float* in_gains = gain_on_input ? (const float*)gains : nullptr;
     const float* out_gains = gain_on_input ? nullptr : (const float*)gains;
     if (form == MOE_PLAIN_RELU2)
         moe_gate_up_kernel<T, MOE_PLAIN_RELU2><<<g1, 256, 0, stream>>>((const T*)x, (const int32_t*)ids,
-                                                                         (const T*)gate_up, in_gains, (T*)act, top, F, K, E);
+                                                                         (const T*)gate_up, in_gains, (T*)act, top, F, K, E, limit);
+    else if (form == MOE_GATED_CLAMP)
+        moe_gate_up_kernel<T, MOE_GATED_CLAMP><<<g1, 256, 0, stream>>>((const T*)x, (const int32_t*)ids,
+                                                                         (const T*)gate_up, in_gains, (T*)act, top, F, K, E, limit);
     else
         moe_gate_up_kernel<T, MOE_GATED_SILU><<<g1, 256, 0, stream>>>((const T*)x, (const int32_t*)ids,
-                                                                        (const T*)gate_up, in_gains, (T*)act, top, F, K, E);
+                                                                        (const T*)gate_up, in_gains, (T*)act, top, F, K, E, limit);
     moe_down_kernel<T><<<g2, 256, 0, stream>>>((const T*)act, (const int32_t*)ids, out_gains, (const T*)down,
                                                 (const T*)x, (float*)out, top, F, H, E);
 }
@@ -289,14 +334,14 @@ static void moe_experts_pairs(const void* x, const void* ids, const void* gains,
 // multiply the experts' inputs, not their results
 extern "C" int lle_moe_experts(const void* x, const void* ids, const void* gains, const void* gate_up,
                                const void* down, void* act, void* out, int N, int top, int E, int F, int K, int H,
-                               int dtype, int form, int gain_on_input, hipStream_t stream) {
+                               int dtype, int form, int gain_on_input, float limit, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (top <= 0 || (int64_t)N * top > 0x7fffffff || form < 0 || form > 1) return (int)hipErrorInvalidValue;
+    if (top <= 0 || (int64_t)N * top > 0x7fffffff || form < 0 || form > 2) return (int)hipErrorInvalidValue;
     if ((F + 3) / 4 > 65535 || (H + 3) / 4 > 65535) return (int)hipErrorInvalidValue;
     if (dtype == LLE_F32)
-        moe_experts_pairs<float>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, stream);
+        moe_experts_pairs<float>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, limit, stream);
     else
-        moe_experts_pairs<bf16_t>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, stream);
+        moe_experts_pairs<bf16_t>(x, ids, gains, gate_up, down, act, out, N, top, E, F, K, H, form, gain_on_input, limit, stream);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -472,7 +517,7 @@ __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* 
                                                                 const bf16_t* __restrict__ gate_up,
                                                                 const float* __restrict__ in_gains,
                                                                 bf16_t* __restrict__ act, int E, int top, int F, int K,
-                                                                int tiles, int blocks) {
+                                                                int tiles, int blocks, float limit) {
     MoeTile t;
     int tile, block;
     if (!moe_grid_item(tiles, blocks, tile, block) || !moe_find_tile(plan, E, tile, t)) return;
@@ -529,7 +574,7 @@ __global__ __launch_bounds__(256, 2) void moe_gate_up_tile_kernel(const bf16_t* 
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float g = gain * acc[half][mt][i], u = gain * acc[2 + half][mt][i];
-                v[i] = (bf16_t)(g / (1.0f + expf(-g)) * u);
+                v[i] = (bf16_t)moe_gated_act<FORM>(g, u, limit);
             }
             *(mbf16x4*)(act + (int64_t)(t.row0 + row) * F + f) = v;
         }
@@ -606,10 +651,10 @@ extern "C" int lle_moe_tile_rows(void) { return MOE_TM; }
 extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void* gains, const void* gate_up,
                                      const void* down, void* plan, void* order, void* place, void* act, void* y,
                                      void* out, int N, int top, int E, int F, int K, int H, int form, int gain_on_input,
-                                     hipStream_t stream) {
+                                     float limit, hipStream_t stream) {
     if (N <= 0) return 0;
     const int64_t pairs64 = (int64_t)N * top;
-    if (top <= 0 || E <= 0 || E > 256 || K % 8 || F % 8 || H % 4 || pairs64 > 0x3fffffff || form < 0 || form > 1)
+    if (top <= 0 || E <= 0 || E > 256 || K % 8 || F % 8 || H % 4 || pairs64 > 0x3fffffff || form < 0 || form > 2)
         return (int)hipErrorInvalidValue;
     const float* in_gains = gain_on_input ? (const float*)gains : nullptr;
     const float* out_gains = gain_on_input ? nullptr : (const float*)gains;
@@ -624,11 +669,15 @@ extern "C" int lle_moe_experts_tiled(const void* x, const void* ids, const void*
     if (form == MOE_PLAIN_RELU2)
         moe_gate_up_tile_kernel<MOE_PLAIN_RELU2><<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
             (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, in_gains, (bf16_t*)act,
-            E, top, F, K, tiles, fb);
+            E, top, F, K, tiles, fb, limit);
+    else if (form == MOE_GATED_CLAMP)
+        moe_gate_up_tile_kernel<MOE_GATED_CLAMP><<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
+            (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, in_gains, (bf16_t*)act,
+            E, top, F, K, tiles, fb, limit);
     else
         moe_gate_up_tile_kernel<MOE_GATED_SILU><<<8 * ((tiles * fb + 7) / 8), 256, 0, stream>>>(
             (const bf16_t*)x, (const int32_t*)plan, (const int32_t*)order, (const bf16_t*)gate_up, in_gains, (bf16_t*)act,
-            E, top, F, K, tiles, fb);
+            E, top, F, K, tiles, fb, limit);
     moe_down_tile_kernel<<<8 * ((tiles * hb + 7) / 8), 256, 0, stream>>>(
         (const bf16_t*)act, (const int32_t*)plan, (const bf16_t*)down, (float*)y, E, F, H, tiles, hb);
     moe_gather_kernel<<<N, 256, 0, stream>>>((const float*)y, (const int32_t*)place, out_gains,

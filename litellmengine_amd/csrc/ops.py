@@ -13,7 +13,7 @@ import torch
 from ..parts.base import PartialSums, Prenormed
 from . import build
 from .tuning import ProductTuning
-from .limits import MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH, MAX_WKV_HEAD_DIM
+from .limits import MAX_DELTA_HEAD_DIM, MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH, MAX_WKV_HEAD_DIM
 
 F32, BF16 = 0, 1
 _P = ctypes.c_void_p
@@ -855,11 +855,13 @@ class HipOps:
                          cu_tokens, kv_lens, token_seq, sink, window: Optional[int], scale: float, max_q_len: int,
                          max_kv_len: int, out_dtype) -> torch.Tensor:
         """All heads of every token against the cached latents: q_lat [N, H, rank] (float32 or the
-        cache's type; any strides over N and H), q_rot float32 [N, H, rot], sink float32 [H] ->
+        cache's type; any strides over N and H), q_rot float32 [N, H, rot], sink float32 [H] (None: an ordinary
+        softmax, nothing but the keys in its sum) ->
         sum_j p_j c_j, [N, H, rank] in the cache's type.  `max_q_len` and `max_kv_len` are host-side
         bounds; they choose kernels, never results."""
         _dev(q_rot, "q_rot", torch.float32)
-        _dev(sink, "sink", torch.float32)
+        if sink is not None:
+            _dev(sink, "sink", torch.float32)
         for t, name in ((block_table, "block_table"), (seq_slots, "seq_slots"), (cu_tokens, "cu_tokens"),
                         (kv_lens, "kv_lens"), (token_seq, "token_seq")):
             _dev(t, name, torch.int32)
@@ -867,7 +869,7 @@ class HipOps:
         S = seq_slots.shape[0]
         _need(q_lat.is_cuda and q_lat.shape == (N, H, rank) and q_lat.stride(2) == 1, "q_lat must be [N, H, rank]")
         _need(q_lat.dtype in (torch.float32, pages.dtype), "q_lat is float32 or of the cache's type")
-        _need(q_rot.shape == (N, H, rot) and sink.shape == (H,), "q_rot [N, H, rot], sink [H]")
+        _need(q_rot.shape == (N, H, rot) and (sink is None or sink.shape == (H,)), "q_rot [N, H, rot], sink [H]")
         _need(pages.is_cuda and pages.dim() == 2 and pages.stride(1) == 1 and pages.dtype == out_dtype
               and pages.shape[1] >= page_size * (2 * rank + rot), "pages must be [pages, page_size * (2 rank + rot)]")
         _need(token_seq.shape == (N,) and cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "the step's arrays")
@@ -922,31 +924,41 @@ class HipOps:
                   _ptr(gains), N, E, top, cols, 1 if score == "sigmoid" else 0)
         return ids, gains
 
-    def moe_route_grouped(self, logits, correction, top: int, groups: int = 1, keep: int = 1):
+    def moe_route_grouped(self, logits, correction, top: int, groups: int = 1, keep: int = 1, score: str = "softmax",
+                          group_top: int = 1):
         """float32 logits [N, E] -> (int32 ids [N, top], float32 gains [N, top]).  Scores are the softmax over
-        all E; the choice is made on score + correction [E], among the experts of the `keep` of `groups` equal
-        groups of neighbours whose largest choice score is largest (the lower index wins a tie); gains are the
-        chosen scores, without the correction, divided by their sum (+ 1e-20)."""
+        all E (`score` "sigmoid": every logit's own sigmoid); the choice is made on score + correction [E] (None:
+        on the scores), among the experts of the `keep` of `groups` equal groups of neighbours whose `group_top`
+        largest choice scores add up to most (the lower index wins a tie); gains are the chosen scores, without
+        the correction, divided by their sum (+ 1e-20)."""
         _dev(logits, "router logits", torch.float32)
-        _dev(correction, "router correction", torch.float32)
         N, E = logits.shape
-        _need(correction.shape == (E,) and 0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
+        if correction is not None:
+            _dev(correction, "router correction", torch.float32)
+            _need(correction.shape == (E,), "the router's correction must be [E]")
+        _need(score in ("softmax", "sigmoid") and group_top >= 1, f"unknown router score {score!r}")
+        _need(0 < top <= min(E, 32), "a router picks between 1 and 32 of its experts")
         _need(groups > 0 and E % groups == 0 and 0 < keep <= groups and top <= keep * (E // groups),
               "the experts form equal groups, and the kept groups hold at least `top` experts")
         _need(2 * E + groups <= 4096, "the router's kernel keeps its scores in LDS: at most about 2000 experts")
         ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
         gains = torch.empty((N, top), dtype=torch.float32, device=logits.device)
-        self._run("moe", "lle_moe_route_grouped", [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P], _ptr(logits),
-                  _ptr(correction), _ptr(ids), _ptr(gains), N, E, top, int(groups), int(keep))
+        self._run("moe", "lle_moe_route_grouped", [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P], _ptr(logits),
+                  _ptr(correction), _ptr(ids), _ptr(gains), N, E, top, int(groups), int(keep),
+                  1 if score == "sigmoid" else 0, int(group_top))
         return ids, gains
 
     MOE_TILED_MIN_PAIRS = 129  # (token, choice) pairs from which the sorted, tiled kernels take a bfloat16 step
 
-    def moe_experts(self, x, ids, gains, gate_up, down, form: str = "gated_silu", gain_on_input: bool = False) -> torch.Tensor:
+    EXPERT_FORMS = {"gated_silu": 0, "relu2": 1, "gated_clamp": 2}
+
+    def moe_experts(self, x, ids, gains, gate_up, down, form: str = "gated_silu", gain_on_input: bool = False,
+                    limit: float = 0.0) -> torch.Tensor:
         """x [N, K]; ids, gains [N, top]; gate_up [E, 2 F, K] (gate rows, then up rows); down [E, H, F] ->
         float32 [N, H]: sum_k gains[n, k] * down[e] (silu(gate[e] x) * (up[e] x)), e = ids[n, k].  An id from E on
         names an identity expert, whose result is x itself (then H = K).
         `form` "relu2": experts without a gate, down[e] relu(up[e] x)^2, `gate_up` is up [E, F, K].
+        `form` "gated_clamp": g = min(gate[e] x, limit), u = clamp(up[e] x, -limit, limit), down[e] (g sigmoid(1.702 g) (u + 1)).
         `gain_on_input`: the result is sum_k expert_e(gains[n, k] * x) instead; the gain is applied to the first
         products' results, in 32-bit, before the activation.
         Few pairs, or float32: every pair streams its expert's rows.  Many bfloat16 pairs: sorted by expert
@@ -958,7 +970,8 @@ class HipOps:
         _dev(down, "down", x.dtype)
         N, K = x.shape
         top = ids.shape[1]
-        _need(form in ("gated_silu", "relu2"), f"unknown expert form {form!r}")
+        _need(form in self.EXPERT_FORMS, f"unknown expert form {form!r}")
+        _need(form != "gated_clamp" or limit > 0.0, "clamped experts need a positive limit")
         plain = form == "relu2"
         E, F2, _ = gate_up.shape
         H = down.shape[1]
@@ -967,29 +980,30 @@ class HipOps:
         _need(gate_up.shape == (E, F2, K) and (plain or F2 % 2 == 0) and down.shape == (E, H, F), "expert weights do not fit")
         act = torch.empty((N * top, F), dtype=x.dtype, device=x.device)
         out = torch.empty((N, H), dtype=torch.float32, device=x.device)
-        code, on_input = (1 if plain else 0), (1 if gain_on_input else 0)
+        code, on_input = self.EXPERT_FORMS[form], (1 if gain_on_input else 0)
         if (x.dtype == torch.bfloat16 and N * top >= self.MOE_TILED_MIN_PAIRS and E <= 256 and K % 8 == 0 and F % 8 == 0
                 and H % 4 == 0):
             plan = torch.empty((4 * E + 1,), dtype=torch.int32, device=x.device)
             order = torch.empty((2, N * top), dtype=torch.int32, device=x.device)
             y = torch.empty((N * top, H), dtype=torch.float32, device=x.device)
             self._run("moe", "lle_moe_experts_tiled",
-                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
                       _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(plan), order[0].data_ptr(),
-                      order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H, code, on_input)
+                      order[1].data_ptr(), _ptr(act), _ptr(y), _ptr(out), N, top, E, F, K, H, code, on_input, float(limit))
             return out
-        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+        self._run("moe", "lle_moe_experts", [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
                   _ptr(x), _ptr(ids), _ptr(gains), _ptr(gate_up), _ptr(down), _ptr(act), _ptr(out), N, top, E, F,
-                  K, H, dtype_code(x.dtype), code, on_input)
+                  K, H, dtype_code(x.dtype), code, on_input, float(limit))
         return out
 
     # -- projections normed as a whole, sinks' attention gates -------------------------------
     def proj_norm_rope_write(self, qkv, bias, slots, q_weight, k_weight, cos_sin, rotary_dim: int, eps: float, kv_layer,
                              num_q_heads: int, num_kv_heads: int, dim: int, vdim: int, has_kv: bool = True,
-                             write_kv: bool = True) -> torch.Tensor:
+                             write_kv: bool = True, per_head: bool = False) -> torch.Tensor:
         """A row of qkv holds q [nq dim], then (`has_kv`) k [nkv dim] and v [nkv vdim], then columns that are
         left alone; `bias` (or None) covers the whole row.  q and k are divided by the root mean square of their
-        whole projection, times q_weight [nq dim] / k_weight [nkv dim], then the first `rotary_dim` elements of
+        whole projection (`per_head`: every head by its own), times q_weight [nq dim] / k_weight [nkv dim] (None:
+        times one), then the first `rotary_dim` elements of
         every head are rotated (half-split) by cos_sin [N, rotary_dim / 2, 2].  Returns q [N, nq, D] with
         D = kv_layer.shape[4] >= max(dim, vdim), zeros past dim; K and V^T go to the pages `kv_layer`
         [pages, 2, nkv, page_size, D] at `slots` [N] with zeros past dim and vdim."""
@@ -1008,21 +1022,25 @@ class HipOps:
         if bias is not None:
             _dev(bias, "bias", qkv.dtype)
             _need(bias.shape == (cols,), "bias must cover the whole row")
-        _dev(q_weight, "q norm weight")
-        _need(q_weight.shape == (nq * dim,), f"q norm weight must be [{nq * dim}]")
-        if has_kv:
+        if q_weight is not None:
+            _dev(q_weight, "q norm weight")
+            _need(q_weight.shape == (nq * dim,), f"q norm weight must be [{nq * dim}]")
+        if has_kv and k_weight is not None:
+            _need(q_weight is not None, "both norms have weights, or neither")
             _dev(k_weight, "k norm weight", q_weight.dtype)
             _need(k_weight.shape == (nkv * dim,), f"k norm weight must be [{nkv * dim}]")
+        _need(not per_head or nq + nkv <= 512, "heads normed one by one: at most 512 query and key heads together")
         if rotary_dim > 0:
             _dev(cos_sin, "cos_sin", torch.float32)
             _need(cos_sin.shape == (N, rotary_dim // 2, 2), "cos_sin must be [N, rotary_dim / 2, 2]")
         q_out = torch.empty((N, nq, D), dtype=qkv.dtype, device=qkv.device)
         self._run("rope_kv", "lle_proj_norm_rope_write",
-                  [_P, _I, _P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _I, _I, _I, _P],
+                  [_P, _I, _P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _I, _I, _I, _I, _P],
                   _ptr(qkv), cols, _ptr(bias), _ptr(slots), _ptr(q_weight), _ptr(k_weight) if has_kv else None,
-                  dtype_code(q_weight.dtype), _ptr(cos_sin) if rotary_dim > 0 else None, rotary_dim, float(eps),
-                  _ptr(q_out), _ptr(kv_layer), N, nq, nkv, dim, vdim, D, page_size, kv_layer.stride(0),
-                  1 if has_kv else 0, 1 if write_kv else 0, dtype_code(qkv.dtype))
+                  dtype_code(q_weight.dtype) if q_weight is not None else F32, _ptr(cos_sin) if rotary_dim > 0 else None,
+                  rotary_dim, float(eps), _ptr(q_out), _ptr(kv_layer), N, nq, nkv, dim, vdim, D, page_size,
+                  kv_layer.stride(0), 1 if has_kv else 0, 1 if write_kv else 0, 1 if per_head else 0,
+                  dtype_code(qkv.dtype))
         return q_out
 
     def head_gate(self, a, gates, col0: int, heads: int, vdim: int) -> torch.Tensor:
@@ -1130,11 +1148,11 @@ class HipOps:
         return out
 
     # -- activations, caps, chained norms ---------------------------------------------------------
-    ACT_CODES = {"silu": 0, "relu": 1, "relu2": 2}
+    ACT_CODES = {"silu": 0, "relu": 1, "relu2": 2, "gelu_tanh": 3}
 
     def bias_act(self, z, kind: str, gated: bool, bias=None, row_gate=None) -> torch.Tensor:
         """gated: z [N, 2 F] (gate columns first) -> act(gate + b) * (up + b), [N, F]; else z [N, F] -> act(z + b).
-        `kind`: silu, relu, relu2 (the square of relu); `bias` (or None) covers z's row; `row_gate` = (t, col), t
+        `kind`: silu, relu, relu2 (the square of relu), gelu_tanh (gelu in its tanh form); `bias` (or None) covers z's row; `row_gate` = (t, col), t
         float32 [N, any]: row n is multiplied by sigmoid(t[n, col]).  Everything in 32-bit."""
         _dev(z, "z")
         _need(kind in self.ACT_CODES, f"unknown activation {kind!r}")
@@ -1245,6 +1263,88 @@ class HipOps:
         _need(kept > 0 and state.shape[1] >= kept * cols and cu_tokens.shape == (S + 1,), "a state row holds `kept` rows of u")
         self._run("rope_kv", "lle_conv_state_update", [_P, _I, _P, _L, _I, _P, _P, _I, _I, _P], _ptr(u), cols, _ptr(state),
                   state.stride(0), int(kept), _ptr(cu_tokens), _ptr(seq_slots), S, dtype_code(u.dtype))
+
+    # -- the gated delta rule --------------------------------------------------------------
+    DELTA_MAX_DIM = MAX_DELTA_HEAD_DIM
+
+    def delta_conv(self, u, taps, state, token_seq, cu_tokens, seq_slots, kv_heads: int, dim: int, heads: int, vdim: int,
+                   unit_eps: float, q_scale: float):
+        """A row of u holds q [G dim], k [G dim], v [H vdim] of one token (G = kv_heads, H = heads).  Every channel is
+        convolved over time with its J taps (float32 [cols, J]; the last tap meets the token itself), reading the
+        rows of the same request ahead of it in this step and, before those, the request's state row (float32
+        [slots + 1, >= (J - 1) cols], the last J - 1 rows of u that earlier steps brought, oldest first; None for
+        J = 1), then passes silu; every head of q and k becomes x / sqrt(sum x^2 + unit_eps), q times q_scale.
+        Returns float32 q [N, G dim], k [N, G dim], v [N, H vdim].  The state is left as it is: conv_state_update
+        advances it."""
+        _dev(u, "u")
+        _dev(taps, "taps", torch.float32)
+        for t, name in ((token_seq, "token_seq"), (cu_tokens, "cu_tokens"), (seq_slots, "seq_slots")):
+            _dev(t, name, torch.int32)
+        N, cols = u.shape
+        J = taps.shape[1]
+        S = seq_slots.shape[0]
+        G, H = int(kv_heads), int(heads)
+        _need(cols == 2 * G * dim + H * vdim, "a row of u holds q, k and v")
+        _need(taps.shape == (cols, J) and J >= 1, "taps must be [cols, J]")
+        _need(token_seq.shape == (N,) and cu_tokens.shape == (S + 1,), "token_seq [N]; cu_tokens [S + 1]")
+        _need(0 < dim <= self.DELTA_MAX_DIM and 0 < vdim <= self.DELTA_MAX_DIM,
+              f"a head of the delta rule holds at most {self.DELTA_MAX_DIM} channels")
+        if J > 1:
+            _need(state is not None, "a convolution of several taps needs the requests' state rows")
+            _rows(state, "state", torch.float32)
+            _need(state.shape[1] >= (J - 1) * cols, "a state row holds J - 1 rows of u")
+        q = torch.empty((N, G * dim), dtype=torch.float32, device=u.device)
+        k = torch.empty((N, G * dim), dtype=torch.float32, device=u.device)
+        v = torch.empty((N, H * vdim), dtype=torch.float32, device=u.device)
+        self._run("delta", "lle_delta_conv", [_P, _I, _P, _I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _I, _P],
+                  _ptr(u), cols, _ptr(taps), J, _ptr(state) if J > 1 else None, state.stride(0) if J > 1 else 0,
+                  _ptr(token_seq), _ptr(cu_tokens), _ptr(seq_slots), _ptr(q), _ptr(k), _ptr(v), N, G, dim, H, vdim,
+                  float(unit_eps), float(q_scale), dtype_code(u.dtype))
+        return q, k, v
+
+    def delta_scan(self, q, k, v, ba, a_log, dt_bias, state, heads: int, kv_heads: int, dim: int, vdim: int, seq_slots,
+                   cu_tokens) -> torch.Tensor:
+        """Per head h, with the matrix state S [dim, vdim] of the request (float32; `state[slot]` holds the heads'
+        states transposed, [heads][vdim][dim]) and the q, k of head h // (heads // kv_heads), token by token:
+            beta = sigmoid(ba[t, h]);  g = exp(-exp(a_log[h]) softplus(ba[t, heads + h] + dt_bias[h]))
+            S <- g S;  w = beta (v_t - S^T k_t);  S <- S + k_t w^T;  o_t = S^T q_t
+        q, k float32 [N, kv_heads dim]; v float32 [N, heads vdim]; ba float32 [N, 2 heads]; a_log, dt_bias float32
+        [heads].  Returns o float32 [N, heads vdim]; the states are advanced in place."""
+        for t, name in ((q, "q"), (k, "k"), (v, "v"), (ba, "ba"), (a_log, "a_log"), (dt_bias, "dt_bias")):
+            _dev(t, name, torch.float32)
+        _rows(state, "state", torch.float32)
+        _dev(seq_slots, "seq_slots", torch.int32)
+        _dev(cu_tokens, "cu_tokens", torch.int32)
+        N = v.shape[0]
+        S = seq_slots.shape[0]
+        H, G = int(heads), int(kv_heads)
+        _need(G > 0 and H % G == 0, "the value heads are a multiple of the query/key heads")
+        _need(0 < dim <= self.DELTA_MAX_DIM, f"a head of the delta rule holds at most {self.DELTA_MAX_DIM} key channels")
+        _need(q.shape == (N, G * dim) and k.shape == (N, G * dim) and v.shape == (N, H * vdim) and ba.shape == (N, 2 * H),
+              "q, k [N, kv_heads dim]; v [N, heads vdim]; ba [N, 2 heads]")
+        _need(a_log.shape == (H,) and dt_bias.shape == (H,), "a_log and dt_bias must be [heads]")
+        _need(state.shape[1] >= H * vdim * dim, "a state row holds heads * vdim * dim floats")
+        _need(cu_tokens.shape == (S + 1,), "cu_tokens must be [S + 1]")
+        out = torch.empty((N, H * vdim), dtype=torch.float32, device=v.device)
+        self._run("delta", "lle_delta_scan", [_P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+                  _ptr(q), _ptr(k), _ptr(v), _ptr(ba), _ptr(a_log), _ptr(dt_bias), _ptr(state), state.stride(0),
+                  _ptr(seq_slots), _ptr(cu_tokens), _ptr(out), S, H, G, dim, vdim)
+        return out
+
+    def delta_out_norm(self, o, gate, norm_w, eps: float, heads: int, vdim: int) -> torch.Tensor:
+        """o float32 [N, heads vdim], gate [N, heads vdim] in the activation type -> every head of o divided by its
+        root mean square (eps inside the root) times norm_w [vdim] times silu(gate), in the gate's type."""
+        _dev(o, "o", torch.float32)
+        _dev(gate, "gate")
+        _dev(norm_w, "norm weight")
+        N = o.shape[0]
+        _need(o.shape == (N, heads * vdim) and gate.shape == o.shape and norm_w.shape == (vdim,),
+              "o and gate [N, heads vdim]; norm weight [vdim]")
+        out = torch.empty_like(gate)
+        self._run("delta", "lle_delta_out_norm", [_P, _P, _P, _I, _F, _P, _I, _I, _I, _I, _P], _ptr(o), _ptr(gate),
+                  _ptr(norm_w), dtype_code(norm_w.dtype), float(eps), _ptr(out), N, int(heads), int(vdim),
+                  dtype_code(gate.dtype))
+        return out
 
     # -- picking tokens --------------------------------------------------------------
     def argmax(self, logits, scatter=None) -> torch.Tensor:

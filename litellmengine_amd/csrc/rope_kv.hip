@@ -415,8 +415,8 @@ extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* slots,
 // Projections normed as a whole.  A row of `qkv` holds q [nq dim], then (with keys and values of
 // its own) k [nkv dim] and v [nkv vdim], then `extra` columns that are left alone; `bias` (or none)
 // covers the whole row.  q and k are divided by the root mean square of their WHOLE projection
-// (all heads at once), times a weight per element, then the first `rot` elements of every head are
-// rotated in the half-split layout.  The cache's heads hold D >= max(dim, vdim) elements: q leaves
+// (all heads at once; `per_head`: of each head on its own), times a weight per element (none: times
+// one), then the first `rot` elements of every head are rotated in the half-split layout.  The cache's heads hold D >= max(dim, vdim) elements: q leaves
 // as [N, nq, D] and K, V^T go to the pages with zeros past dim and vdim.  grid = tokens.
 // ---------------------------------------------------------------------------------
 template <typename T>
@@ -430,15 +430,34 @@ __device__ __forceinline__ float pn_normed_rotated(const T* __restrict__ row, co
                                                    int head, int dim, int e, float inv, const void* __restrict__ weight,
                                                    int wd, const float* __restrict__ cs, int rot) {
     const int at = head * dim + e;
-    const float x = pn_value<T>(row, bias, col0 + at) * inv * load_as_f32(weight, at, wd);
+    const float x = pn_value<T>(row, bias, col0 + at) * inv * (weight ? load_as_f32(weight, at, wd) : 1.0f);
     if (e >= rot) return x;
     const int half = rot / 2;
     const bool low = e < half;
     const int i = low ? e : e - half;
     const int pe = low ? e + half : e - half;
-    const float y = pn_value<T>(row, bias, col0 + head * dim + pe) * inv * load_as_f32(weight, head * dim + pe, wd);
+    const float y = pn_value<T>(row, bias, col0 + head * dim + pe) * inv *
+                    (weight ? load_as_f32(weight, head * dim + pe, wd) : 1.0f);
     const float c = cs[2 * i], s = cs[2 * i + 1];
     return low ? x * c - y * s : x * c + y * s;
+}
+
+#define PN_MAX_HEADS 512  // q heads and kv heads together whose own factors fit the workgroup's LDS
+
+// one factor per head of a projection that starts at column col0: 1 / sqrt(mean of the head's squares + eps)
+template <typename T>
+__device__ __forceinline__ void pn_head_factors(const T* __restrict__ row, const T* __restrict__ bias, int col0, int heads,
+                                                int dim, float eps, float* __restrict__ inv) {
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE, waves = blockDim.x / LLE_WAVE;
+    for (int h = wave; h < heads; h += waves) {
+        float ss = 0.f;
+        for (int e = lane; e < dim; e += LLE_WAVE) {
+            const float x = pn_value<T>(row, bias, col0 + h * dim + e);
+            ss += x * x;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) inv[h] = 1.0f / sqrtf(ss / (float)dim + eps);
+    }
 }
 
 template <typename T>
@@ -446,37 +465,49 @@ __global__ __launch_bounds__(256) void proj_norm_rope_write_kernel(
     const T* __restrict__ qkv, int cols, const T* __restrict__ bias, const int32_t* __restrict__ slots,
     const void* __restrict__ q_weight, const void* __restrict__ k_weight, int wd, const float* __restrict__ cos_sin,
     int rot, float eps, T* __restrict__ q_out, T* __restrict__ kv_layer, int nq, int nkv, int dim, int vdim, int D,
-    int page_size, int64_t page_stride, int has_kv, int write_kv) {
+    int page_size, int64_t page_stride, int has_kv, int write_kv, int per_head) {
     __shared__ float red[16];
+    __shared__ float head_inv[PN_MAX_HEADS];
     const int64_t n = blockIdx.x;
     const T* row = qkv + n * cols;
     const float* cs = cos_sin + n * rot;  // [rot / 2][2]
     const int qw = nq * dim, kw = nkv * dim;
-    float ss = 0.f;
-    for (int e = threadIdx.x; e < qw; e += blockDim.x) {
-        const float x = pn_value<T>(row, bias, e);
-        ss += x * x;
+    float inv_q = 0.f, inv_k = 0.f;
+    if (per_head) {
+        pn_head_factors<T>(row, bias, 0, nq, dim, eps, head_inv);
+        if (has_kv) pn_head_factors<T>(row, bias, qw, nkv, dim, eps, head_inv + nq);
+        __syncthreads();
+    } else {
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < qw; e += blockDim.x) {
+            const float x = pn_value<T>(row, bias, e);
+            ss += x * x;
+        }
+        inv_q = 1.0f / sqrtf(block_sum(ss, red) / (float)qw + eps);
     }
-    const float inv_q = 1.0f / sqrtf(block_sum(ss, red) / (float)qw + eps);
     for (int idx = threadIdx.x; idx < nq * D; idx += blockDim.x) {
         const int h = idx / D, e = idx - h * D;
-        const float y = e < dim ? pn_normed_rotated<T>(row, bias, 0, h, dim, e, inv_q, q_weight, wd, cs, rot) : 0.f;
+        const float inv = per_head ? head_inv[h] : inv_q;
+        const float y = e < dim ? pn_normed_rotated<T>(row, bias, 0, h, dim, e, inv, q_weight, wd, cs, rot) : 0.f;
         q_out[n * nq * D + idx] = from_f32<T>(y);
     }
     if (!has_kv) return;
-    ss = 0.f;
-    for (int e = threadIdx.x; e < kw; e += blockDim.x) {
-        const float x = pn_value<T>(row, bias, qw + e);
-        ss += x * x;
+    if (!per_head) {
+        float ss = 0.f;
+        for (int e = threadIdx.x; e < kw; e += blockDim.x) {
+            const float x = pn_value<T>(row, bias, qw + e);
+            ss += x * x;
+        }
+        inv_k = 1.0f / sqrtf(block_sum(ss, red) / (float)kw + eps);
     }
-    const float inv_k = 1.0f / sqrtf(block_sum(ss, red) / (float)kw + eps);
     const int slot = slots[n];
     if (!write_kv || slot < 0) return;
     const int page = slot / page_size, off = slot - page * page_size;
     T* dst = kv_layer + (int64_t)page * page_stride;
     for (int idx = threadIdx.x; idx < nkv * D; idx += blockDim.x) {
         const int h = idx / D, e = idx - h * D;
-        const float y = e < dim ? pn_normed_rotated<T>(row, bias, qw, h, dim, e, inv_k, k_weight, wd, cs, rot) : 0.f;
+        const float inv = per_head ? head_inv[nq + h] : inv_k;
+        const float y = e < dim ? pn_normed_rotated<T>(row, bias, qw, h, dim, e, inv, k_weight, wd, cs, rot) : 0.f;
         dst[((int64_t)h * page_size + off) * D + e] = from_f32<T>(y);
         const float v = e < vdim ? pn_value<T>(row, bias, qw + kw + h * vdim + e) : 0.f;
         dst[(int64_t)nkv * page_size * D + ((int64_t)h * D + e) * page_size + off] = from_f32<T>(v);
@@ -487,19 +518,20 @@ extern "C" int lle_proj_norm_rope_write(const void* qkv, int cols, const void* b
                                         const void* q_weight, const void* k_weight, int weight_dtype, const void* cos_sin,
                                         int rot, float eps, void* q_out, void* kv_layer, int N, int nq, int nkv, int dim,
                                         int vdim, int D, int page_size, int64_t page_stride, int has_kv, int write_kv,
-                                        int dtype, hipStream_t stream) {
+                                        int per_head, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
     if (rot % 2 || rot > dim || dim > D || vdim > D || (rot > 0 && cos_sin == nullptr)) return (int)hipErrorInvalidValue;
+    if (per_head && nq + nkv > PN_MAX_HEADS) return (int)hipErrorInvalidValue;
     if (dtype == LLE_F32)
         proj_norm_rope_write_kernel<float><<<N, 256, 0, stream>>>(
             (const float*)qkv, cols, (const float*)bias, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
             (const float*)cos_sin, rot, eps, (float*)q_out, (float*)kv_layer, nq, nkv, dim, vdim, D, page_size, page_stride,
-            has_kv, write_kv);
+            has_kv, write_kv, per_head);
     else
         proj_norm_rope_write_kernel<bf16_t><<<N, 256, 0, stream>>>(
             (const bf16_t*)qkv, cols, (const bf16_t*)bias, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
             (const float*)cos_sin, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, dim, vdim, D, page_size,
-            page_stride, has_kv, write_kv);
+            page_stride, has_kv, write_kv, per_head);
     LLE_RETURN_LAUNCH_STATUS();
 }
 

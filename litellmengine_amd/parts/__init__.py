@@ -2,6 +2,7 @@ from .attention import ConvAttention, PagedAttention, SinkAttention
 from .base import (Block, BuildContext, CacheField, Carried, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
                    Normed, PartialSums, PositionEncoding, Prenormed, ScaledSum, StateSpec)
 from .block import ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock
+from .delta import GatedDeltaMixer
 from .embedding import Embedding
 from .feed_forward import GatedMLP, PlainMLP
 from .latent_attention import LatentAttention
@@ -18,5 +19,5 @@ __all__ = [
     "RoutedMLP", "RotaryInterleaved", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
     "NoPositionEncoding", "Norm", "NormFold", "Normed", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec", "GroupLimitedMLP", "ParallelBlock", "ScaledSum", "SinkAttention", "WKVMixer",
-    "ConvAttention", "SandwichBlock", "PlainMLP", "ScoreRoutedMLP", "SideBySideMixer",
+    "ConvAttention", "SandwichBlock", "PlainMLP", "ScoreRoutedMLP", "SideBySideMixer", "GatedDeltaMixer",
 ]

@@ -150,8 +150,10 @@ class SinkAttention(Mixer):
         q = W_q h + b_q, k = W_k h + b_k, v = W_v h + b_v
         q, k <- divided by the root mean square of the WHOLE projection (all heads at once), times a
                 weight per element; then the position encoding on the first elements of every head
+                (`norm_over="head"`: every head by its own root mean square; `norm_weights=False`: no
+                weight tensors, the division alone)
         p_j = exp(s_j) / (exp(sink) + sum_j exp(s_j)),  s_j = (q . k_j) * scale,  over the last `window` keys
-        out = W_o [heads' (sum_j p_j v_j) * sigmoid(W_g h)_head]
+        out = W_o [heads' (sum_j p_j v_j) * sigmoid(W_g h)_head]        (`gate=False`: no gate, no W_g)
 
     Keys may be `dim` wide and values `vdim`: the cache's heads hold `cache_dim` >= both elements (a
     multiple of 32, which the matrix-core kernels take), the rest zeros, so the kernels of
@@ -166,7 +168,8 @@ class SinkAttention(Mixer):
     def __init__(self, prefix: str, hidden_size: int, num_q_heads: int, num_kv_heads: int, dim: int, vdim: int,
                  position: PositionEncoding, norm_eps: float, scale: float, window: Optional[int] = None,
                  sink: Optional[float] = 0.0, own_kv: bool = True, cache_window=None,
-                 names: Sequence[str] = ("q", "k", "v", "g", "o"), bias_suffix: str = ".b", norm_suffix: str = ".norm"):
+                 names: Sequence[str] = ("q", "k", "v", "g", "o"), bias_suffix: str = ".b", norm_suffix: str = ".norm",
+                 norm_over: str = "projection", norm_weights: bool = True, gate: bool = True):
         if num_q_heads % num_kv_heads:
             raise ValueError("num_q_heads must be a multiple of num_kv_heads")
         self.cache_dim = -(-max(dim, vdim) // 32) * 32
@@ -182,6 +185,9 @@ class SinkAttention(Mixer):
         self.window = window
         self.sink = sink
         self.own_kv = bool(own_kv)
+        if norm_over not in ("projection", "head"):
+            raise ValueError(f"q and k are normed over the whole projection or head by head, not over {norm_over!r}")
+        self.per_head, self.norm_weights, self.gated = norm_over == "head", bool(norm_weights), bool(gate)
         if cache_window is SinkAttention.UNBOUNDED:
             self._cache_window = None
         else:
@@ -196,7 +202,7 @@ class SinkAttention(Mixer):
         w = [(self.q_name, self.nq * self.dim, True)]
         if self.own_kv:
             w += [(self.k_name, self.nkv * self.dim, True), (self.v_name, self.nkv * self.vdim, True)]
-        return w + [(self.g_name, self.nq, False)]  # (name, rows, has a bias)
+        return w + ([(self.g_name, self.nq, False)] if self.gated else [])  # (name, rows, has a bias)
 
     def cache_spec(self) -> CacheSpec:
         return KVCacheSpec(self.nkv, self.cache_dim, self._cache_window)
@@ -207,9 +213,10 @@ class SinkAttention(Mixer):
             specs[name] = TensorSpec((rows, self.hidden), INIT_NORMAL)
             if biased:
                 specs[name + self.bias_suffix] = TensorSpec((rows,), INIT_NORMAL)
-        specs[self.q_name + self.norm_suffix] = TensorSpec((self.nq * self.dim,), INIT_NORM)
-        if self.own_kv:
-            specs[self.k_name + self.norm_suffix] = TensorSpec((self.nkv * self.dim,), INIT_NORM)
+        if self.norm_weights:
+            specs[self.q_name + self.norm_suffix] = TensorSpec((self.nq * self.dim,), INIT_NORM)
+            if self.own_kv:
+                specs[self.k_name + self.norm_suffix] = TensorSpec((self.nkv * self.dim,), INIT_NORM)
         return specs
 
     def bind(self, weights, ctx: BuildContext) -> None:
@@ -222,8 +229,10 @@ class SinkAttention(Mixer):
             weights[name + self.bias_suffix].to(ctx.dtype).reshape(-1) if biased
             else torch.zeros(rows, dtype=ctx.dtype, device=ctx.device)
             for name, rows, biased in self._widths()]).contiguous()
-        self.q_norm_w = weights[self.q_name + self.norm_suffix].float().contiguous()
-        self.k_norm_w = weights[self.k_name + self.norm_suffix].float().contiguous() if self.own_kv else None
+        self.q_norm_w = self.k_norm_w = None
+        if self.norm_weights:
+            self.q_norm_w = weights[self.q_name + self.norm_suffix].float().contiguous()
+            self.k_norm_w = weights[self.k_name + self.norm_suffix].float().contiguous() if self.own_kv else None
         self.sinks = None if self.sink is None else torch.full((self.nq,), float(self.sink), dtype=torch.float32,
                                                                device=ctx.device)
 
@@ -235,12 +244,16 @@ class SinkAttention(Mixer):
         qkvg = ops.linear(x, self.weight)
         cos_sin, rot = self.position.fused_rotary(step)
         q = ops.proj_norm_rope_write(qkvg, self.bias, group.slot_mapping, self.q_norm_w, self.k_norm_w, cos_sin, rot,
-                                     self.eps, cache.kv, self.nq, self.nkv, self.dim, self.vdim, self.own_kv, cache.writes)
+                                     self.eps, cache.kv, self.nq, self.nkv, self.dim, self.vdim, self.own_kv, cache.writes,
+                                     per_head=self.per_head)
         a = ops.paged_attention(q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens,
                                 step.token_seq, self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
                                 sinks=self.sinks)
-        gated = ops.head_gate(a, qkvg, qkvg.shape[1] - self.nq, self.nq, self.vdim)
-        return self.o.forward(gated)
+        if self.gated:
+            return self.o.forward(ops.head_gate(a, qkvg, qkvg.shape[1] - self.nq, self.nq, self.vdim))
+        if self.cache_dim != self.vdim:  # the attention hands out heads of cache_dim elements: the first vdim of each
+            a = a.view(a.shape[0], self.nq, self.cache_dim)[:, :, : self.vdim].reshape(a.shape[0], self.nq * self.vdim)
+        return self.o.forward(a)
 
 
 class ConvAttention(Mixer):

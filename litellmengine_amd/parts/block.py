@@ -1,25 +1,30 @@
 """Pre-norm residual block: r = x + mixer(norm_in(x)); y = r + ff(norm_post(r))
 (src/model/qwen3.cpp:948-968).  The adds run inside the norm kernels on the
-32-bit residual stream; the last add of a block is left to the next norm."""
+32-bit residual stream; the last add of a block is left to the next norm.  A block
+without a feed-forward is the first line alone: the mixer's result is what it leaves."""
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
+
+import torch
 
 from ..weights.spec import TensorSpec
-from typing import Optional
 
 from .base import Block, BuildContext, Carried, FeedForward, Mixer, Norm, Normed, Prenormed, ScaledSum
 
 
 class PreNormBlock(Block):
-    def __init__(self, norm_in: Norm, mixer: Mixer, norm_post: Norm, feed_forward: FeedForward):
+    def __init__(self, norm_in: Norm, mixer: Mixer, norm_post: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None):
+        if (norm_post is None) != (feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.norm_in = norm_in
         self.mixer = mixer
         self.norm_post = norm_post
         self.feed_forward = feed_forward
 
     def _parts(self):
-        return (self.norm_in, self.mixer, self.norm_post, self.feed_forward)
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_post, self.feed_forward) if p is not None)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs: Dict[str, TensorSpec] = {}
@@ -47,6 +52,8 @@ class PreNormBlock(Block):
             x = delta.x
         else:
             x = self.norm_in.forward(hidden, delta)
+        if self.feed_forward is None:
+            return self.mixer.forward(x, step, cache)
         fold = self.norm_post.fold(hidden) if self.mixer.folds_norm and self.feed_forward.folds_norm else None
         if fold is not None:
             x = self.mixer.forward(x, step, cache, fold=fold)
@@ -55,7 +62,12 @@ class PreNormBlock(Block):
         fold = next_norm.fold(hidden) if next_norm is not None and self.feed_forward.folds_norm else None
         if fold is not None:
             return self.feed_forward.forward(x, fold=fold)
-        return self.feed_forward.forward(x)
+        y = self.feed_forward.forward(x)
+        if isinstance(y, torch.Tensor) and y.dtype != self.ctx.dtype:
+            # a sum that a routed feed-forward has kept in 32-bit enters the stream as it is: the norm's kernel
+            # that takes a sum of sublayers takes either type
+            return ScaledSum(y, None, 1.0)
+        return y
 
 
 class PostNormBlock(Block):

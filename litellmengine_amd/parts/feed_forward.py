@@ -20,10 +20,10 @@ class GatedMLP(FeedForward):
         """`names`: the checkpoint's names of the gate, up and down weights after `prefix`.
         `to_residual`: the result goes nowhere but into Norm.forward(hidden, delta) (it may then
         come as PartialSums); an arrangement that does anything else with it says False.
-        `activation`: silu or relu.  `bias_names`: the three projections' biases after `prefix`
+        `activation`: silu, relu or gelu_tanh (gelu in its tanh form).  `bias_names`: the three projections' biases after `prefix`
         (none: no biases); the gate's and up's are added inside the activation's kernel."""
-        if activation not in ("silu", "relu"):
-            raise ValueError(f"a gated feed-forward's activation is silu or relu, not {activation!r}")
+        if activation not in ("silu", "relu", "gelu_tanh"):
+            raise ValueError(f"a gated feed-forward's activation is silu, relu or gelu_tanh, not {activation!r}")
         self.activation = activation
         biased = bool(bias_names)
         if biased and len(bias_names) != 3:

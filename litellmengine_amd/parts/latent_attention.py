@@ -6,8 +6,11 @@ and only that vector (and one rotated key part shared by the heads) is cached.
                                        k_rot = rotated(second part)  (one for all heads)
     per head: k_plain = W_uk c, v = W_uv c
     score = (q_plain . k_plain + q_rot . k_rot) * scale
-    softmax over the keys AND one sink per head: the denominator also holds exp(sink_h)
+    softmax over the keys AND one sink per head: the denominator also holds exp(sink_h)  (`sink=False`: the keys alone)
     out = W_o [heads' sum_j p_j v_j]
+
+With `q_rank` the queries pass a latent of their own first, q = W_uq (RMSNorm(W_dq h) * w), and with `head_gate`
+head a's result is multiplied by sigmoid(W_g h)_a, a gate that reads the mixer's input.
 
 Nothing per head is ever made for a cached token.  Since q_plain . (W_uk c) = (W_uk^T q_plain) . c
 and sum_j p_j (W_uv c_j) = W_uv (sum_j p_j c_j), a query is carried into the latent space once
@@ -34,11 +37,16 @@ class LatentAttention(Mixer):
 
     def __init__(self, prefix: str, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
                  scale: float, norm_eps: float, position: RotaryInterleaved, window: Optional[int] = None,
-                 names: Sequence[str] = ("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o")):
+                 names: Sequence[str] = ("q", "dkv", "dkv.norm", "uk", "uv", "sink", "o"), sink: bool = True,
+                 q_rank: Optional[int] = None, q_names: Sequence[str] = ("dq", "dq.norm", "uq"),
+                 head_gate: Optional[str] = None):
         """`position` rotates the first `position.rotary_dim` of the `rot_dim` elements.  `names`: the
         checkpoint's names after `prefix` of the query projection, the down projection to
         [latent | rotated key], the latent's norm weight, the up projections to plain keys and to
-        values, the sinks and the output projection."""
+        values, the sinks and the output projection.  `sink=False`: no sink tensor, an ordinary softmax.
+        `q_rank`: the queries' latent size; then `q_names` are the names of the down projection, the latent's
+        norm weight and the up projection to the heads' queries, and names[0] is not read.  `head_gate`: the name
+        of the projection [heads, hidden] whose sigmoids gate the heads' results (None: no gate)."""
         if position.rotary_dim > rot_dim:
             raise ValueError("the rotation covers more elements than the rotated part has")
         self.prefix = prefix
@@ -47,12 +55,25 @@ class LatentAttention(Mixer):
         self.eps = float(norm_eps)
         self.window = window
         self.position = position
-        q, dkv, dkv_norm, uk, uv, sink, o = (prefix + n for n in names)
-        self.q = Linear([q], hidden_size, [heads * (dim + rot_dim)])
+        q, dkv, dkv_norm, uk, uv, sink_name, o = (prefix + n for n in names)
+        self.q_rank = None if q_rank is None else int(q_rank)
+        self.has_sink = bool(sink)
+        if self.q_rank is None:
+            self.q = Linear([q], hidden_size, [heads * (dim + rot_dim)])
+            self.dq = self.q_norm_name = None
+        else:
+            dq, dq_norm, uq = (prefix + n for n in q_names)
+            self.dq = Linear([dq], hidden_size, [self.q_rank])
+            self.q = Linear([uq], self.q_rank, [heads * (dim + rot_dim)])
+            self.q_norm_name = dq_norm
         self.dkv = Linear([dkv], hidden_size, [kv_rank + rot_dim])
+        self.gate = Linear([prefix + head_gate], hidden_size, [heads]) if head_gate else None
         self.o = Linear([o], heads * vdim, [hidden_size])
-        self.norm_name, self.uk_name, self.uv_name, self.sink_name = dkv_norm, uk, uv, sink
-        self.norm_w = self.uk_t = self.uv = self.sink = None
+        self.norm_name, self.uk_name, self.uv_name, self.sink_name = dkv_norm, uk, uv, sink_name
+        self.norm_w = self.uk_t = self.uv = self.sink = self.q_norm_w = None
+
+    def _linears(self):
+        return [p for p in (self.q, self.dq, self.dkv, self.gate, self.o) if p is not None]
 
     def cache_spec(self) -> CacheSpec:
         # the latents twice: token after token for the scores, transposed (the keys of one element
@@ -61,31 +82,41 @@ class LatentAttention(Mixer):
                           CacheField("k_rot", 1, self.rot)), self.window)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {
-            **self.q.tensor_specs(), **self.dkv.tensor_specs(), **self.o.tensor_specs(),
-            self.norm_name: TensorSpec((self.rank,), INIT_NORM),
-            self.uk_name: TensorSpec((self.H * self.dim, self.rank), INIT_NORMAL),
-            self.uv_name: TensorSpec((self.H * self.vdim, self.rank), INIT_NORMAL),
-            self.sink_name: TensorSpec((self.H,), INIT_NORMAL),
-        }
+        specs: Dict[str, TensorSpec] = {}
+        for p in self._linears():
+            specs.update(p.tensor_specs())
+        specs[self.norm_name] = TensorSpec((self.rank,), INIT_NORM)
+        specs[self.uk_name] = TensorSpec((self.H * self.dim, self.rank), INIT_NORMAL)
+        specs[self.uv_name] = TensorSpec((self.H * self.vdim, self.rank), INIT_NORMAL)
+        if self.has_sink:
+            specs[self.sink_name] = TensorSpec((self.H,), INIT_NORMAL)
+        if self.q_norm_name is not None:
+            specs[self.q_norm_name] = TensorSpec((self.q_rank,), INIT_NORM)
+        return specs
 
     def bind(self, weights, ctx: BuildContext) -> None:
         self.ctx = ctx
-        for p in (self.q, self.dkv, self.o, self.position):
+        for p in self._linears() + [self.position]:
             p.bind(weights, ctx)
         self.norm_w = weights[self.norm_name].contiguous()
+        if self.q_norm_name is not None:
+            self.q_norm_w = weights[self.q_norm_name].contiguous()
         # per head, ready for `x . W^T`: W_uk^T [rank, dim] (queries into the latent space) and W_uv [vdim, rank]
         uk = weights[self.uk_name].to(ctx.dtype).view(self.H, self.dim, self.rank)
         self.uk_t = uk.transpose(1, 2).contiguous()
         self.uv = weights[self.uv_name].to(ctx.dtype).view(self.H, self.vdim, self.rank).contiguous()
-        self.sink = weights[self.sink_name].float().contiguous()
+        self.sink = weights[self.sink_name].float().contiguous() if self.has_sink else None
 
     def forward(self, x, step, cache):
         ops = self.ctx.ops
         group = cache.group
         cos_sin = self.position.table(step)
         rot_dims = self.position.rotary_dim
-        q = self.q.forward(x)
+        if self.dq is None:
+            q = self.q.forward(x)
+        else:  # the queries' latent: its norm reads the product's 32-bit result
+            cq = ops.rmsnorm(self.dq.forward(x, out_dtype=torch.float32), self.q_norm_w, self.eps)
+            q = self.q.forward(ops.cast(cq, self.ctx.dtype))
         dkv = self.dkv.forward(x)
         if cache.writes:
             ops.latent_kv_write(dkv, self.norm_w, self.eps, cos_sin, rot_dims, group.slot_mapping, cache.pages,
@@ -99,4 +130,7 @@ class LatentAttention(Mixer):
             step.max_kv_len, self.ctx.dtype,
         )
         v = ops.heads_linear(o_lat, self.H, 0, self.rank, self.uv, self.ctx.dtype)  # [N, H, vdim]
-        return self.o.forward(v.reshape(v.shape[0], self.H * self.vdim))
+        v = v.reshape(v.shape[0], self.H * self.vdim)
+        if self.gate is not None:
+            v = ops.head_gate(v, self.gate.forward(x), 0, self.H, self.vdim)
+        return self.o.forward(v)

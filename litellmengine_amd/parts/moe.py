@@ -82,11 +82,17 @@ class GroupLimitedMLP(FeedForward):
         out = sum_k gains_k * expert_k(h),  expert(h) = down(silu(gate h) * (up h))
 
     The last `identity` router outputs are identity experts: no tensors, their result is h itself.  The
-    experts' weights are stacked, the choice stays on the device, the sum is left in 32-bit."""
+    experts' weights are stacked, the choice stays on the device, the sum is left in 32-bit.
+
+    Parameters for other routers and experts of the same shape: `score="sigmoid"` (s = sigmoid(W_router h), every
+    expert scored on its own), `correction=False` (no correction tensor: c = s), `group_top=n` (a group's score
+    is the sum of its n largest c), `form="gated_clamp"` with `limit` (g = min(gate h, limit),
+    u = clamp(up h, -limit, limit), expert(h) = down(g sigmoid(1.702 g) (u + 1)))."""
 
     def __init__(self, prefix: str, hidden_size: int, expert_size: int, num_experts: int, top: int, identity: int = 0,
                  groups: int = 1, groups_kept: int = 1, expert_prefix: str = "e{}.", names=("gate", "up", "down"),
-                 router_names=("router", "correction")):
+                 router_names=("router", "correction"), score: str = "softmax", correction: bool = True,
+                 group_top: int = 1, form: str = "gated_silu", limit: float = 0.0):
         total = num_experts + identity
         if num_experts <= 0 or identity < 0 or groups <= 0 or total % groups or not 0 < groups_kept <= groups:
             raise ValueError("experts and identity experts together form equal groups, of which some are kept")
@@ -94,15 +100,23 @@ class GroupLimitedMLP(FeedForward):
             raise ValueError("every token uses between one and all of the experts of the kept groups")
         self.prefix, self.hidden, self.ff, self.E, self.identity, self.top = (prefix, hidden_size, expert_size,
                                                                              num_experts, identity, top)
+        if score not in ("softmax", "sigmoid"):
+            raise ValueError(f"a router's scores are a softmax over all experts or sigmoids, not {score!r}")
+        if form not in ("gated_silu", "gated_clamp") or (form == "gated_clamp" and not limit > 0.0):
+            raise ValueError("the experts are gated_silu, or gated_clamp with a positive limit")
+        if group_top < 1:
+            raise ValueError("a group's score adds up at least one of its experts' scores")
         self.groups, self.groups_kept = groups, groups_kept
+        self.score, self.group_top, self.form, self.limit = score, int(group_top), form, float(limit)
         self.expert_names = [[prefix + expert_prefix.format(e) + n for n in names] for e in range(num_experts)]
         self.router = Linear([prefix + router_names[0]], hidden_size, [total])
-        self.correction_name = prefix + router_names[1]
+        self.correction_name = prefix + router_names[1] if correction else None
         self.correction = self.gate_up = self.down = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs = dict(self.router.tensor_specs())
-        specs[self.correction_name] = TensorSpec((self.E + self.identity,), INIT_NORMAL)
+        if self.correction_name is not None:
+            specs[self.correction_name] = TensorSpec((self.E + self.identity,), INIT_NORMAL)
         for gate, up, down in self.expert_names:
             specs[gate] = TensorSpec((self.ff, self.hidden), INIT_NORMAL)
             specs[up] = TensorSpec((self.ff, self.hidden), INIT_NORMAL)
@@ -112,7 +126,8 @@ class GroupLimitedMLP(FeedForward):
     def bind(self, weights, ctx: BuildContext) -> None:
         self.ctx = ctx
         self.router.bind(weights, ctx)
-        self.correction = weights[self.correction_name].float().contiguous()
+        if self.correction_name is not None:
+            self.correction = weights[self.correction_name].float().contiguous()
         self.gate_up = torch.stack(
             [torch.cat([weights[g].to(ctx.dtype), weights[u].to(ctx.dtype)], dim=0) for g, u, _ in self.expert_names]
         ).contiguous()
@@ -121,8 +136,10 @@ class GroupLimitedMLP(FeedForward):
     def forward(self, x):
         ops = self.ctx.ops
         logits = self.router.forward(x, out_dtype=torch.float32)
-        ids, gains = ops.moe_route_grouped(logits, self.correction, self.top, self.groups, self.groups_kept)
-        return ops.moe_experts(x, ids, gains, self.gate_up, self.down)  # float32 [N, hidden]; ids from E on: x itself
+        ids, gains = ops.moe_route_grouped(logits, self.correction, self.top, self.groups, self.groups_kept,
+                                           score=self.score, group_top=self.group_top)
+        # float32 [N, hidden]; ids from E on: x itself
+        return ops.moe_experts(x, ids, gains, self.gate_up, self.down, form=self.form, limit=self.limit)
 
 
 class ScoreRoutedMLP(FeedForward):

@@ -256,6 +256,9 @@ class TorchOps:
                 c = c_pages[pg, off].to(self.cd)  # [n, rank]
                 kr = r_pages[pg, off].to(self.cd)
                 sc = (q_lat[t].to(self.cd) @ c.T + q_rot[t].to(self.cd) @ kr.T) * scale  # [H, n]
+                if sink is None:
+                    out[t] = torch.softmax(sc, dim=1) @ c
+                    continue
                 sk = sink.to(self.cd)[:, None]
                 m = torch.maximum(sc.max(dim=1, keepdim=True).values, sk)
                 e = torch.exp(sc - m)
@@ -273,12 +276,12 @@ class TorchOps:
         gains = torch.sigmoid(vals) if score == "sigmoid" else torch.softmax(vals, dim=-1)
         return idx.to(torch.int32), gains.to(torch.float32)
 
-    def moe_route_grouped(self, logits, correction, top, groups=1, keep=1):
-        s = torch.softmax(logits.to(self.cd), dim=-1)
-        c = s + correction.to(self.cd)
+    def moe_route_grouped(self, logits, correction, top, groups=1, keep=1, score="softmax", group_top=1):
+        s = torch.sigmoid(logits.to(self.cd)) if score == "sigmoid" else torch.softmax(logits.to(self.cd), dim=-1)
+        c = s if correction is None else s + correction.to(self.cd)
         N, E = c.shape
         size = E // groups
-        best = c.view(N, groups, size).max(dim=-1).values
+        best = torch.sort(c.view(N, groups, size), dim=-1, descending=True).values[:, :, :group_top].sum(-1)
         # (a stable sort: among equal scores the lower index comes first, for groups and for experts)
         kept = torch.sort(best, dim=-1, descending=True, stable=True).indices[:, :keep]
         allowed = torch.zeros((N, groups), dtype=torch.bool, device=c.device).scatter_(1, kept, True)
@@ -287,8 +290,8 @@ class TorchOps:
         chosen = torch.gather(s, 1, ids)
         return ids.to(torch.int32), (chosen / (chosen.sum(-1, keepdim=True) + 1e-20)).to(torch.float32)
 
-    def moe_experts(self, x, ids, gains, gate_up, down, form="gated_silu", gain_on_input=False):
-        if form != "gated_silu" or gain_on_input:
+    def moe_experts(self, x, ids, gains, gate_up, down, form="gated_silu", gain_on_input=False, limit=0.0):
+        if form == "relu2" or gain_on_input:
             return self._moe_experts_plain(x, ids, gains, gate_up, down, form, gain_on_input)
         N, top = ids.shape
         ff = gate_up.shape[1] // 2
@@ -301,7 +304,11 @@ class TorchOps:
                     out[n] += gains[n, k].to(self.cd) * xx[n]
                     continue
                 gu = gate_up[e].to(self.cd) @ xx[n]
-                a = gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]
+                if form == "gated_clamp":
+                    g, u = torch.clamp(gu[:ff], max=limit), torch.clamp(gu[ff:], min=-limit, max=limit)
+                    a = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+                else:
+                    a = gu[:ff] * torch.sigmoid(gu[:ff]) * gu[ff:]
                 a = a.to(x.dtype).to(self.cd)
                 out[n] += gains[n, k].to(self.cd) * (down[e].to(self.cd) @ a)
         return out.to(torch.float32)
@@ -327,7 +334,8 @@ class TorchOps:
         if bias is not None:
             zz = zz + bias.to(self.cd)
         act = {"silu": lambda t: t * torch.sigmoid(t), "relu": lambda t: torch.clamp(t, min=0.0),
-               "relu2": lambda t: torch.clamp(t, min=0.0) ** 2}[kind]
+               "relu2": lambda t: torch.clamp(t, min=0.0) ** 2,
+               "gelu_tanh": lambda t: 0.5 * t * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (t + 0.044715 * t ** 3)))}[kind]
         if gated:
             F = zz.shape[1] // 2
             out = act(zz[:, :F]) * zz[:, F:]
@@ -408,7 +416,7 @@ class TorchOps:
 
     # -- projections normed as a whole, gates per head, side-by-side sublayers -------------------
     def proj_norm_rope_write(self, qkv, bias, slots, q_weight, k_weight, cos_sin, rotary_dim, eps, kv_layer,
-                             num_q_heads, num_kv_heads, dim, vdim, has_kv=True, write_kv=True):
+                             num_q_heads, num_kv_heads, dim, vdim, has_kv=True, write_kv=True, per_head=False):
         nq, nkv = num_q_heads, num_kv_heads
         N = qkv.shape[0]
         D, P = kv_layer.shape[4], kv_layer.shape[3]
@@ -417,7 +425,12 @@ class TorchOps:
             x = x + bias.to(self.cd)
 
         def norm(t, w):
-            return t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps) * w.to(self.cd)
+            if per_head:
+                h = t.reshape(N, -1, dim)
+                t = (h / torch.sqrt((h * h).mean(-1, keepdim=True) + eps)).reshape(N, -1)
+            else:
+                t = t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps)
+            return t if w is None else t * w.to(self.cd)
 
         def rope(t):
             if rotary_dim == 0:
@@ -443,6 +456,62 @@ class TorchOps:
                 kv_layer[page, 0, :, off, :] = k[n].to(kv_layer.dtype)
                 v_pages(kv_layer)[page, :, :, off] = v[n].to(kv_layer.dtype)
         return q.to(qkv.dtype).contiguous()
+
+    # -- the gated delta rule ------------------------------------------------------------------
+    def delta_conv(self, u, taps, state, token_seq, cu_tokens, seq_slots, kv_heads, dim, heads, vdim, unit_eps, q_scale):
+        N, cols = u.shape
+        J = taps.shape[1]
+        G, H = kv_heads, heads
+        y = torch.zeros((N, cols), dtype=self.cd, device=u.device)
+        for s in range(seq_slots.shape[0]):
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 <= q0:
+                continue
+            rows = u[q0:q1].to(self.cd)
+            if J > 1:
+                kept = state[int(seq_slots[s]), : (J - 1) * cols].view(J - 1, cols).to(self.cd)
+                rows = torch.cat([kept, rows], dim=0)
+            for j in range(J):
+                y[q0:q1] += rows[j : j + (q1 - q0)] * taps[:, j].to(self.cd)
+        y = y * torch.sigmoid(y)
+
+        def unit(t):
+            h = t.reshape(N, G, dim)
+            return (h / torch.sqrt((h * h).sum(-1, keepdim=True) + unit_eps)).reshape(N, G * dim)
+
+        q = unit(y[:, : G * dim]) * q_scale
+        k = unit(y[:, G * dim : 2 * G * dim])
+        return q.to(torch.float32), k.to(torch.float32), y[:, 2 * G * dim :].to(torch.float32).contiguous()
+
+    def delta_scan(self, q, k, v, ba, a_log, dt_bias, state, heads, kv_heads, dim, vdim, seq_slots, cu_tokens):
+        N = v.shape[0]
+        H, G = heads, kv_heads
+        out = torch.zeros((N, H, vdim), dtype=self.cd, device=v.device)
+        qq, kk, vv = q.to(self.cd).view(N, G, dim), k.to(self.cd).view(N, G, dim), v.to(self.cd).view(N, H, vdim)
+        beta = torch.sigmoid(ba[:, :H].to(self.cd))
+        g = torch.exp(-torch.exp(a_log.to(self.cd)) * torch.nn.functional.softplus(ba[:, H:].to(self.cd) + dt_bias.to(self.cd)))
+        for s in range(seq_slots.shape[0]):
+            q0, q1 = int(cu_tokens[s]), int(cu_tokens[s + 1])
+            if q1 <= q0:
+                continue
+            slot = int(seq_slots[s])
+            S = state[slot, : H * vdim * dim].view(H, vdim, dim).to(self.cd).clone()  # [head][value][key]
+            for t in range(q0, q1):
+                for h in range(H):
+                    j = h // (H // G)
+                    S[h] = g[t, h] * S[h]
+                    w = beta[t, h] * (vv[t, h] - S[h] @ kk[t, j])
+                    S[h] = S[h] + torch.outer(w, kk[t, j])
+                    out[t, h] = S[h] @ qq[t, j]
+            state[slot, : H * vdim * dim] = S.reshape(-1).to(state.dtype)
+        return out.reshape(N, H * vdim).to(torch.float32)
+
+    def delta_out_norm(self, o, gate, norm_w, eps, heads, vdim):
+        N = o.shape[0]
+        x = o.to(self.cd).view(N, heads, vdim)
+        x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * norm_w.to(self.cd)
+        gg = gate.to(self.cd).view(N, heads, vdim)
+        return (x * gg * torch.sigmoid(gg)).reshape(N, heads * vdim).to(gate.dtype)
 
     def head_gate(self, a, gates, col0, heads, vdim):
         N = a.shape[0]
