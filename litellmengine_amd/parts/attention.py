@@ -221,7 +221,12 @@ class SinkAttention(Mixer):
 
     def bind(self, weights, ctx: BuildContext) -> None:
         self.ctx = ctx
-        self.o.bind(weights, ctx)
+        if self.gated or self.cache_dim == self.vdim:
+            self.o.bind(weights, ctx)
+        else:  # without gates nothing drops the cache's padding: the output projection gets zero columns there
+            o = weights[self.o.names[0]].to(ctx.dtype)
+            o = torch.nn.functional.pad(o.view(self.hidden, self.nq, self.vdim), (0, self.cache_dim - self.vdim))
+            self.o.bind_tensor(o.reshape(self.hidden, self.nq * self.cache_dim).contiguous(), ctx)
         self.position.bind(weights, ctx)
         # one product for q, (k, v,) and the gates' inputs; the gates have no bias
         self.weight = torch.cat([weights[name].to(ctx.dtype) for name, _, _ in self._widths()], dim=0).contiguous()
@@ -249,11 +254,9 @@ class SinkAttention(Mixer):
         a = ops.paged_attention(q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens,
                                 step.token_seq, self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
                                 sinks=self.sinks)
-        if self.gated:
+        if self.gated:  # (the gates' kernel also drops the cache's padding)
             return self.o.forward(ops.head_gate(a, qkvg, qkvg.shape[1] - self.nq, self.nq, self.vdim))
-        if self.cache_dim != self.vdim:  # the attention hands out heads of cache_dim elements: the first vdim of each
-            a = a.view(a.shape[0], self.nq, self.cache_dim)[:, :, : self.vdim].reshape(a.shape[0], self.nq * self.vdim)
-        return self.o.forward(a)
+        return self.o.forward(a)  # heads of cache_dim elements, zeros past vdim, against zero columns of the weight
 
 
 class ConvAttention(Mixer):

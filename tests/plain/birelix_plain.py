@@ -68,7 +68,8 @@ def rotate_neighbours(x: torch.Tensor, positions: torch.Tensor, dims: int, base:
 def latent_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict, eps: float,
                  positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     T = h.shape[0]
-    H, dim, rot, vdim, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    H, dim, rot, vdim = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+    rank = w[p + "dkv.norm"].shape[0]  # the latent's size (config `kv_rank`, where it says it)
     pos = torch.arange(T) if positions is None else positions
     rdims, base = m["rot"]["dims"], m["rot"]["base"]
     cq = rms_norm(h @ w[p + "dq"].T, w[p + "dq.norm"], eps)
