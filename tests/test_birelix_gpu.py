@@ -1,0 +1,190 @@
+"""Birelix on the GPU: bin/trace_run as a child process (whole prompts, decoded tails, portions
+down to two tokens, mixed batches in a pool of the live peak with four slots) in float32 and
+bfloat16 against the plain model, with weights made so that single keys, the windows' edges, the
+softmax's extra place, the convolutions' taps, the delta states' memory and the routers' choices
+carry the result; every layer's residual stream; long decoding through captured graphs with a slot
+used again; generation through the Python entry point and the command line."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests.birelix_util import CONFIGS, PAGE_SIZES, make_model_dir, plain_logits, read, residual_streams, run_tool, sharpen
+from tests.plain import birelix_plain as plain
+from tests.tiny import random_tokens
+from tests.trace_util import ROOT, TraceBuilder, changing_portions, check_dumps, mixed, tail_one_by_one, whole
+
+pytestmark = pytest.mark.gpu
+
+# About five times the worst error seen.  With scores sharpened and gates, routers and the delta rule's beta and
+# decay projections grown, the rounding of their bfloat16 inputs alone moves the logits by tenths (the same
+# arithmetic on the CPU with bfloat16 storage shows it too): the bfloat16 runs leave those as they are and pin
+# gross faults; what is exact is pinned by the float32 runs.
+TOL = {"float32": 2e-4, "bfloat16": 1e-1}
+SHARP = {"float32": 3.0, "bfloat16": 1.0}
+GENTLE = {"float32": (), "bfloat16": (".mix.g", ".mlp.router", ".mix.b", ".mix.a")}
+LENGTHS = {"a": 70, "b": 45, "c": 100, "d": 33, "e": 64, "f": 1, "g": 2}
+
+
+def all_ways_trace(requests, tail=32):
+    tb = TraceBuilder()
+    names = list(requests)
+    whole(tb, names[0] + "#whole", requests[names[0]])
+    whole(tb, names[2] + "#whole", requests[names[2]])
+    tail_one_by_one(tb, names[1] + "#tail", requests[names[1]], tail=tail)
+    changing_portions(tb, names[2] + "#cut", requests[names[2]], seed=1)
+    changing_portions(tb, names[4] + "#cut", requests[names[4]], seed=2)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=5)
+    return tb
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "A/default page", "B", "C"])
+def test_trace_gpu(tmp_path, which, dtype):
+    which, default_page = which[0], len(which) > 1
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    sharpen(d, SHARP[dtype], same_experts=dtype == "bfloat16", skip=GENTLE[dtype])
+    vocab = CONFIGS[which]["vocab"]
+    requests = {rid: random_tokens(n, vocab, 10 + i) for i, (rid, n) in enumerate(LENGTHS.items())}
+    tb = all_ways_trace(requests)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=None if default_page else PAGE_SIZES[which])
+    worst = check_dumps(out, tb, plain_logits(d, requests), TOL[dtype])
+    print(f"trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_one_layer_at_a_time_follows_the_plain_model_gpu(tmp_path, which, dtype):
+    """The residual stream after every block: a whole prompt, then the same prompt in two portions and three
+    single tokens through the cache and the state rows (so the first layer that goes wrong is named)."""
+    from litellmengine_amd.cache import CacheManager
+    from litellmengine_amd.engine import ModelRunner, StepEntry
+    from litellmengine_amd.models import load_model
+
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    sharpen(d, SHARP[dtype], same_experts=dtype == "bfloat16", skip=GENTLE[dtype])
+    tokens = random_tokens(70, CONFIGS[which]["vocab"], 3)
+    want = residual_streams(d, tokens)
+    model = load_model(d, dtype)
+    cache = CacheManager(model, page_size=PAGE_SIZES[which], num_pages=40, max_requests=2, dtype=model.ctx.dtype,
+                         device=model.ctx.device)
+    runner = ModelRunner(model, cache, use_graphs=False)
+    seen = []
+    for b in model.blocks:
+        def wrapped(hidden, delta, step, layer_cache, next_norm=None, inner=b.forward):
+            out = inner(hidden, delta, step, layer_cache, next_norm=next_norm)
+            h = hidden.double().cpu()
+            if out is not None:  # what the block leaves to be added by whoever comes next
+                h = h + (out.total() if hasattr(out, "total") else out).double().cpu()
+            seen.append(h)
+            return out
+        b.forward = wrapped
+    tol = 2e-4 if dtype == "float32" else 6e-2
+    for cuts in ([70], [40, 27, 1, 1, 1]):
+        slot, at = runner.admit(), 0
+        for n in cuts:
+            seen.clear()
+            runner.step([StepEntry(slot, tokens[at : at + n], [])])
+            for i, (got, ref) in enumerate(zip(seen, want)):
+                err = (got - ref[at : at + n]).abs().max() / ref.abs().max()
+                assert err < tol, f"layer {i}, tokens {at}..{at + n}: {float(err):.3g}"
+            at += n
+        runner.release(slot)
+    for b in model.blocks:
+        del b.forward  # (the wrappers hold the model in a cycle)
+
+
+# Larger scores carry the rounding of queries and keys further into the softmax weights: the tolerances
+# grow with the factor.
+PEAK = {("A", "float32"): (5.0, 2e-3), ("A", "bfloat16"): (1.5, 2e-1),
+        ("B", "float32"): (6.0, 2e-3), ("B", "bfloat16"): (1.5, 2e-1)}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_trace_with_single_keys_standing_out(tmp_path, which, dtype):
+    """Requests of hundreds of tokens whose latent attention picks out single keys, near and hundreds back, whose
+    windows pass over prompt portions and decoded tokens (keys just inside and just outside them), whose delta
+    states remember for hundreds of tokens in some heads and whose routers choose clearly; the last 80 tokens of
+    one request are decoded one by one."""
+    d = make_model_dir(tmp_path, which, seed=5, dtype=torch.bfloat16)
+    factor, tol = PEAK[which, dtype]
+    sharpen(d, factor, same_experts=dtype == "bfloat16", memory=1.6, skip=GENTLE[dtype])
+    vocab = CONFIGS[which]["vocab"]
+    requests = {"p": random_tokens(300, vocab, 41), "q": random_tokens(170, vocab, 42),
+                "r": random_tokens(230, vocab, 43), "s": random_tokens(90, vocab, 44)}
+    tb = TraceBuilder()
+    whole(tb, "p#whole", requests["p"])
+    tail_one_by_one(tb, "p#tail", requests["p"], tail=80)
+    changing_portions(tb, "r#cut", requests["r"], seed=3)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=6)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=PAGE_SIZES[which])
+    worst = check_dumps(out, tb, plain_logits(d, requests), tol)
+    print(f"peaked trace {which} {dtype}: worst relative error {worst:.3g}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_in_a_batch_with_slots_used_again(tmp_path, dtype):
+    """Three requests decode 150 tokens each side by side (captured graphs), the shortest ends and its
+    slot, pages and state rows go to a newcomer whose prompt runs beside the others' single tokens."""
+    d = make_model_dir(tmp_path, "B", seed=9, dtype=torch.bfloat16)
+    sharpen(d, 4.0 if dtype == "float32" else 1.0, same_experts=dtype == "bfloat16", memory=1.6, skip=GENTLE[dtype])
+    vocab = CONFIGS["B"]["vocab"]
+    requests = {rid: random_tokens(n, vocab, 60 + i) for i, (rid, n) in enumerate({"a": 170, "b": 200, "c": 230, "n": 90}.items())}
+    tb = TraceBuilder()
+    tb.step([(r, requests[r][: len(requests[r]) - 150], [0]) for r in "abc"])
+    live, at = ["a", "b", "c"], {r: len(requests[r]) - 150 for r in "abc"}
+    at["n"] = 0
+    for i in range(150):
+        entries, end = [], []
+        for r in list(live):
+            n = 40 if r == "n" and at[r] == 0 else 1
+            entries.append((r, requests[r][at[r] : at[r] + n], [n - 1]))
+            at[r] += n
+            if at[r] == len(requests[r]):
+                end.append(r)
+                live.remove(r)
+        tb.step(entries, end)
+        if i == 20:
+            live.remove("a")
+            tb.steps[-1]["end"].append("a")
+            tb.live.pop("a")
+            live.append("n")
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=16, max_requests=3)
+    worst = check_dumps(out, tb, plain_logits(d, requests), 2e-3 if dtype == "float32" else 1.5e-1)
+    print(f"long decoding {dtype}: worst relative error {worst:.3g}")
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(tmp_path, which):
+    from litellmengine_amd.entrypoints.generate import generate
+
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    sharpen(d, 2.0)
+    cfg, w = read(d)
+    prompts = [random_tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate((1, 7, 23, 60))]
+    want = [plain.greedy(cfg, w, p, 12) for p in prompts]
+    assert generate(d, prompts, max_tokens=12, dtype="float32", page_size=PAGE_SIZES[which]) == want
+    # portions, and a pool in which requests are preempted and recomputed
+    assert generate(d, prompts, max_tokens=12, dtype="float32", page_size=8, prefill_chunk=16,
+                    max_tokens_per_step=24, num_pages=14) == want
+
+
+def test_command_line_generates(tmp_path):
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    sharpen(d, 2.0)
+    cfg, w = read(d)
+    prompt = random_tokens(19, cfg["vocab"], 80)
+    want = plain.greedy(cfg, w, prompt, 10)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "litellmengine"), "--model", d, "--input-ids",
+                           ",".join(map(str, prompt)), "--max-tokens", "10", "--temperature", "0", "--dtype", "float32"],
+                          text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.split("\n")
+    got = [int(t) for t in lines[lines.index("New token ids:") + 1].replace(" ", "").split(",")]
+    assert got == want
