@@ -11,6 +11,7 @@
     python bench.py --workload visadra [--sizes small|mid|wide]   # Visadra beside Qwen3 at equal layer sizes, kernel by kernel
     python bench.py --workload kezasun [--sizes small|mid|wide]   # Kezasun beside Visadra, kernel by kernel
     python bench.py --workload malilorn [--sizes small|mid|wide]  # Malilorn beside Kezasun, kernel by kernel
+    python bench.py --workload birelix [--sizes small|mid|wide]   # Birelix beside Kezasun, kernel by kernel
 
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
@@ -943,6 +944,201 @@ def malilorn_workload(args):
     return 0
 
 
+BIRELIX_SIZES = {
+    # width; latent: heads, dim, rotated, vdim, kv rank, q rank; window attention: q heads, kv heads, dim, vdim, window;
+    # delta: value heads, query/key heads, dim, vdim, taps; experts, top, expert ff, groups, kept, limit; dense ff
+    "small": (1024, 8, 128, 64, 128, 512, 768, 8, 2, 128, 128, 1024, 16, 8, 64, 64, 4, 16, 4, 512, 4, 2, 7.0, 4096),
+    "mid": (2048, 16, 128, 64, 128, 512, 1536, 16, 4, 128, 128, 2048, 32, 16, 64, 64, 4, 64, 6, 1408, 8, 4, 7.0, 8192),
+    "wide": (4096, 32, 128, 64, 128, 512, 1536, 32, 8, 128, 128, 4096, 64, 32, 64, 64, 4, 64, 6, 2048, 8, 4, 7.0, 12288),
+}
+
+
+def birelix_config(which, groups):
+    from litellmengine_amd.config import BirelixConfig
+
+    (W, LH, ldim, lrot, lvdim, rank, qrank, H, G, dim, vdim, window, DH, DG, ddim, dvdim, taps, E, top, eff, ng, keep, limit,
+     ff) = BIRELIX_SIZES[which]
+    lat = {"heads": LH, "dim": ldim, "rot_dim": lrot, "vdim": lvdim, "kv_rank": rank, "q_rank": qrank,
+           "scale": (ldim + lrot) ** -0.5, "rot": {"base": 250000.0, "dims": lrot}}
+    att = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "mask": {"size": window}}
+    dlt = {"heads": DH, "kv_heads": DG, "dim": ddim, "vdim": dvdim, "conv": taps}
+    moe = {"kind": "moe", "expert": {"ff": eff, "limit": limit}, "router": {"experts": E, "top": top, "groups": {"count": ng, "keep": keep}}}
+    four = [{"type": "latent_attention", "mixer": lat, "mlp": {"kind": "dense", "ff": ff}}, {"type": "delta", "mixer": dlt, "mlp": moe},
+            {"type": "latent_attention", "mixer": lat, "mlp": moe}, {"type": "attention", "mixer": att, "mlp": moe}]
+    return BirelixConfig.from_dict({"architecture": "Birelix", "vocab": 32768, "width": W, "embedding": {"scale": W ** 0.5},
+                                    "norm": {"eps": 1e-6}, "layers": four * groups})
+
+
+def birelix_kernels(which):
+    """Each kernel of Birelix's own at two shapes (a 2048-token prompt; 8 decoded tokens after 4096) beside the
+    like kernel of Kezasun (the closest model: a recurrence with a matrix state per head, grouped-query attention
+    over a window with a sink, experts chosen among the best groups) at its sizes of the same name, or of Visadra
+    for the latent attention: microseconds and the share of its roofline."""
+    import torch
+
+    from litellmengine_amd.csrc.ops import default_ops
+
+    ops = default_ops()
+    (W, LH, ldim, lrot, lvdim, rank, qrank, H, G, dim, vdim, window, DH, DG, ddim, dvdim, taps, E, top, eff, ng, keep, limit,
+     ff) = BIRELIX_SIZES[which]
+    KW, kwh, kwd, krank, KH, KG, kdim, kvdim, krot, kwindow, KE, KI, ktop, keff, kng, kkeep = KEZASUN_SIZES[which]
+    dev, bf = "cuda", torch.bfloat16
+    P = PAGE_SIZE
+    rnd = lambda *shape, dtype=bf, scale=1.0: (torch.randn(shape, device=dev) * scale).to(dtype)
+    ints = lambda values: torch.tensor(values, dtype=torch.int32, device=dev)
+    out = {}
+
+    def entry(name, seconds, flops, nbytes, like=None):
+        floor = max(flops / MFMA_PEAK["bf16"], nbytes / HBM_PEAK)
+        e = {"us": round(seconds * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "frac": round(floor / seconds, 4),
+             "bound": "mfma" if flops / MFMA_PEAK["bf16"] > nbytes / HBM_PEAK else "hbm"}
+        if like is not None:
+            e["like"] = like
+            e["times_farther_from_roofline"] = round(like["frac"] / e["frac"], 2) if e["frac"] > 0 else None
+        out[name] = e
+        return e
+
+    for shape, S, q_len, past in (("prefill_2048", 1, 2048, 0), ("decode_b8_ctx4096", 8, 1, 4095)):
+        N, kv = S * q_len, past + q_len
+        pages_each = -(-kv // P)
+        table = torch.arange(S * pages_each, dtype=torch.int32, device=dev).view(S, pages_each).contiguous()
+        seq_slots, cu = ints(list(range(S))), ints([i * q_len for i in range(S + 1)])
+        kv_lens = ints([kv] * S)
+        token_seq = ints([i // q_len for i in range(N)])
+        slots = (table.long().repeat_interleave(P, 1)[:, past:kv] * P + torch.arange(past, kv, device=dev) % P).reshape(-1).int()
+        # the delta rule's walk beside the walk of the recurrence with a decayed matrix state
+        q, k = rnd(N, DG * ddim, dtype=torch.float32, scale=ddim ** -0.5), rnd(N, DG * ddim, dtype=torch.float32, scale=ddim ** -0.5)
+        v, ba = rnd(N, DH * dvdim, dtype=torch.float32), rnd(N, 2 * DH, dtype=torch.float32)
+        a_log = dt_bias = torch.zeros(DH, device=dev)
+        dstate = torch.zeros(S + 1, DH * dvdim * ddim, device=dev)
+        t = timed_launches(lambda: ops.delta_scan(q, k, v, ba, a_log, dt_bias, dstate, DH, DG, ddim, dvdim, seq_slots, cu))
+        HD = kwh * kwd
+        r, kk, vv, wraw = (rnd(N, HD, dtype=torch.float32, scale=0.5) for _ in range(4))
+        w0 = u0 = torch.zeros(HD, device=dev)
+        g, x = rnd(N, HD), rnd(N, KW)
+        kstate = torch.zeros(S + 1, HD * kwd + KW, device=dev)
+        tk = timed_launches(lambda: ops.wkv_scan(r, kk, vv, wraw, w0, u0, g, torch.ones(HD, device=dev), 1e-6, x, kstate, kwh, kwd,
+                                                 seq_slots, cu, bf, q_len))
+        like = entry(f"{shape}/wkv_scan (Kezasun)", tk, 0, N * HD * (16 + 2 + 2.0) + 2.0 * S * HD * kwd * 4)
+        e = entry(f"{shape}/delta_scan", t, 0, N * (2 * DG * ddim + 2 * DH * dvdim + 2 * DH) * 4.0 + 2.0 * S * DH * dvdim * ddim * 4,
+                  dict(like, name="wkv_scan"))
+        e["fp32_flops_T"] = round(8.0 * N * DH * dvdim * ddim / t / 1e12, 2)
+        # the output norm with its gate (the recurrence beside it does this in its walk's epilogue) beside the gates per head
+        o, gate, nw = rnd(N, DH * dvdim, dtype=torch.float32), rnd(N, DH * dvdim), torch.ones(dvdim, device=dev)
+        t = timed_launches(lambda: ops.delta_out_norm(o, gate, nw, 1e-6, DH, dvdim))
+        KD = -(-max(kdim, kvdim) // 32) * 32
+        a, gates = rnd(N, KH * KD), rnd(N, KH)
+        tk = timed_launches(lambda: ops.head_gate(a, gates, 0, KH, kvdim))
+        like = entry(f"{shape}/head_gate (Kezasun)", tk, 0, 2.0 * N * (KH * KD + KH * kvdim))
+        entry(f"{shape}/delta_out_norm", t, 0, N * DH * dvdim * (4 + 2 + 2.0), dict(like, name="head_gate"))
+        # the convolution with silu and unit vectors (and the kept rows' update) beside the mixes of neighbouring tokens
+        cols = 2 * DG * ddim + DH * dvdim
+        uu, conv_w = rnd(N, cols), rnd(cols, taps, dtype=torch.float32)
+        cstate = torch.zeros(S + 1, (taps - 1) * cols, device=dev)
+
+        def conv():
+            ops.delta_conv(uu, conv_w, cstate, token_seq, cu, seq_slots, DG, ddim, DH, dvdim, 1e-6, ddim ** -0.5)
+            ops.conv_state_update(uu, cstate, taps - 1, cu, seq_slots)
+
+        t = timed_launches(conv)
+        mu = rnd(5, KW, dtype=torch.float32)
+        tk = timed_launches(lambda: ops.shift_mix(x, kstate, HD * kwd, mu, token_seq, cu, seq_slots))
+        like = entry(f"{shape}/shift_mix (Kezasun)", tk, 0, 2.0 * N * KW * 6)
+        entry(f"{shape}/delta_conv + conv_state_update", t, 0, N * cols * (2 + 4.0) + 8.0 * S * (taps - 1) * cols,
+              dict(like, name="shift_mix"))
+        # q and k normed head by head (biases, no weights, no rotation) with the cache write beside the norm over whole projections
+        D = -(-max(dim, vdim) // 32) * 32
+        kv_layer = rnd(S * pages_each + 1, 2, G, P, D)
+        pcols = H * dim + G * (dim + vdim)
+        qkv, bias = rnd(N, pcols), rnd(pcols)
+        t = timed_launches(lambda: ops.proj_norm_rope_write(qkv, bias, slots, None, None, None, 0, 1e-6, kv_layer, H, G, dim, vdim,
+                                                            per_head=True))
+        kkv = rnd(S * pages_each + 1, 2, KG, P, KD)
+        kcols = KH * kdim + KG * (kdim + kvdim) + KH
+        kqkv, kbias = rnd(N, kcols), rnd(kcols)
+        kqw, kkw = torch.ones(KH * kdim, device=dev), torch.ones(KG * kdim, device=dev)
+        positions = ints([past + i % q_len for i in range(N)])
+        kcs = ops.rope_table(positions, torch.ones(krot // 2, device=dev))
+        tk = timed_launches(lambda: ops.proj_norm_rope_write(kqkv, kbias, slots, kqw, kkw, kcs, krot, 1e-6, kkv, KH, KG, kdim, kvdim))
+        like = entry(f"{shape}/proj_norm_rope_write (Kezasun)", tk, 0, 2.0 * N * (kcols + KH * KD + 2 * KG * KD))
+        entry(f"{shape}/proj_norm_rope_write, head by head", t, 0, 2.0 * N * (pcols + H * D + 2 * G * D),
+              dict(like, name="proj_norm_rope_write"))
+        # latent attention with an ordinary softmax beside the same kernel with sinks
+        lat_pages = rnd(S * pages_each + 1, P * (2 * rank + lrot))
+        q_lat, q_rot = rnd(LH, N, rank, scale=0.1).transpose(0, 1), rnd(N, LH, lrot, dtype=torch.float32, scale=0.1)
+        args = (q_lat, q_rot, lat_pages, P, rank, lrot, table, seq_slots, cu, kv_lens, token_seq)
+        t = timed_launches(lambda: ops.latent_attention(*args, None, None, 0.1, q_len, kv, bf))
+        vsink = torch.zeros(LH, device=dev)
+        tv = timed_launches(lambda: ops.latent_attention(*args, vsink, None, 0.1, q_len, kv, bf))
+        visible = S * (q_len * past + q_len * (q_len + 1) / 2)
+        fl, by = 2.0 * LH * (2 * rank + lrot) * visible, 2.0 * (S * kv * (2 * rank + lrot) + 2 * N * LH * rank)
+        like = entry(f"{shape}/latent_attention with sinks (Visadra)", tv, fl, by)
+        entry(f"{shape}/latent_attention, ordinary softmax", t, fl, by, dict(like, name="latent_attention"))
+        # the routers and the experts
+        logits = rnd(N, E, dtype=torch.float32)
+        t = timed_launches(lambda: ops.moe_route_grouped(logits, None, top, ng, keep, score="sigmoid", group_top=2))
+        klogits, kcorr = rnd(N, KE + KI, dtype=torch.float32), torch.zeros(KE + KI, device=dev)
+        tk = timed_launches(lambda: ops.moe_route_grouped(klogits, kcorr, ktop, kng, kkeep))
+        like = entry(f"{shape}/moe_route_grouped (Kezasun)", tk, 0, N * (4.0 * (KE + KI) + 8 * ktop))
+        entry(f"{shape}/moe_route_grouped, sigmoid scores, groups by their two largest", t, 0, N * (4.0 * E + 8 * top),
+              dict(like, name="moe_route_grouped"))
+        xx = rnd(N, W, scale=0.1)
+        gu, down = rnd(E, 2 * eff, W, scale=0.02), rnd(E, W, eff, scale=0.02)
+        ids, gains = ops.moe_route_grouped(logits, None, top, ng, keep, score="sigmoid", group_top=2)
+        t = timed_launches(lambda: ops.moe_experts(xx, ids, gains, gu, down, form="gated_clamp", limit=limit), repeats=5)
+        kx = rnd(N, KW, scale=0.1)
+        kgu, kdown = rnd(KE, 2 * keff, KW, scale=0.02), rnd(KE, KW, keff, scale=0.02)
+        kids, kgains = ops.moe_route_grouped(klogits, kcorr, ktop, kng, kkeep)
+        tk = timed_launches(lambda: ops.moe_experts(kx, kids, kgains, kgu, kdown), repeats=5)
+        real = int((kids < KE).sum())
+        like = entry(f"{shape}/moe_experts with identity experts (Kezasun)", tk, 6.0 * real * KW * keff,
+                     2.0 * (3 * min(KE, real) * KW * keff + 2 * N * KW))
+        entry(f"{shape}/moe_experts, clamped", t, 6.0 * N * top * W * eff, 2.0 * (3 * min(E, N * top) * W * eff + 2 * N * W),
+              dict(like, name="moe_experts"))
+        # the dense feed-forward's activation beside silu_mul
+        z2 = rnd(N, 2 * ff)
+        t = timed_launches(lambda: ops.bias_act(z2, "gelu_tanh", True))
+        ts = timed_launches(lambda: ops.silu_mul(z2))
+        like = entry(f"{shape}/silu_mul (Qwen3)", ts, 0, 2.0 * N * 3 * ff)
+        entry(f"{shape}/bias_act, gated tanh-gelu", t, 0, 2.0 * N * 3 * ff, dict(like, name="silu_mul"))
+        del kv_layer, kkv, lat_pages
+    return out
+
+
+def birelix_workload(args):
+    import torch
+
+    from litellmengine_amd.models import random_model
+
+    which = args.sizes if args.sizes in BIRELIX_SIZES else "mid"
+    groups = max(1, args.layers // 4) if args.layers != SIZES["num_hidden_layers"] else 2
+    bcfg = birelix_config(which, groups)
+    kcfg = kezasun_config(which, groups)
+    names = ("width", "latent_heads", "latent_dim", "latent_rotated", "latent_vdim", "kv_rank", "q_rank", "heads", "kv_heads", "dim",
+             "vdim", "window", "delta_heads", "delta_kv_heads", "delta_dim", "delta_vdim", "taps", "experts", "top", "expert_ff",
+             "groups", "kept", "limit", "dense_ff")
+    line = {"metric": f"Birelix beside Kezasun at layer sizes of the same name ({which}): prefill tok/s @ 2048 and decode tok/s "
+                      f"@ batch {args.batch}, context {args.context}", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+            "data": "synthetic: seeded random weights, uniform random token ids", "higher_is_better": True,
+            "config": {"sizes": dict(zip(names, BIRELIX_SIZES[which])), "layers": 4 * groups,
+                       "pattern": "latent+dense, delta+moe, latent+moe, attention+moe",
+                       "beside": f"Kezasun with {4 * groups} layers: wkv+moe, attention+moe, wkv+moe, attention+moe"}}
+    steps, warmup = min(args.steps, 16), min(args.warmup, 4)
+    for name, cfg in (("birelix", bcfg), ("kezasun", kcfg)):
+        model = random_model(cfg, seed=0, dtype="bfloat16")
+        dt = time_decode(model, cfg, args.batch, args.context, steps, warmup)
+        pt = time_prefill(model, cfg, PREFILL_TOKENS)
+        line[name] = {"decode_tok_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                      "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
+        del model
+        torch.cuda.empty_cache()
+    line["value"] = line["birelix"]["decode_tok_s"]
+    line["steps"], line["warmup"] = steps, warmup
+    line["kernels"] = birelix_kernels(which)
+    print(json.dumps(line))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -956,12 +1152,12 @@ def main():
     ap.add_argument("--no-more", action="store_true", help="skip the other workloads that the default line carries")
     ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b", "small", "mid", "wide"],
                     help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B; "
-                         "small, mid or wide: the layer sizes of --workload visadra, kezasun and malilorn")
-    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra", "kezasun", "malilorn"],
+                         "small, mid or wide: the layer sizes of --workload visadra, kezasun, malilorn and birelix")
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving", "visadra", "kezasun", "malilorn", "birelix"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
                          "sizes, a mixed prompt-portion + decode step at Qwen3-32B sizes, requests arriving over time, "
                          "Visadra beside Qwen3 at equal layer sizes with every kernel against its roofline, Kezasun "
-                         "beside Visadra the same way, or Malilorn beside Kezasun the same way")
+                         "beside Visadra the same way, or Malilorn or Birelix beside Kezasun the same way")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
@@ -981,6 +1177,8 @@ def main():
             return kezasun_workload(args)
         if args.workload == "malilorn":
             return malilorn_workload(args)
+        if args.workload == "birelix":
+            return birelix_workload(args)
         args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
         return mixed_workload(args)
 

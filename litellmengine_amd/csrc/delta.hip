@@ -19,9 +19,10 @@
 LLE_DEFINE_ERROR_STRING()
 
 #define DELTA_IG 16   // threads that share a column of the state
-#define DELTA_TC 8    // tokens staged at a time
+#define DELTA_TC 16   // tokens staged at a time
 #define DELTA_THREADS 256
 #define DELTA_VB (DELTA_THREADS / DELTA_IG)  // value channels of a workgroup
+static_assert(DELTA_VB == DELTA_TC, "the walk's kernel deals the staged tokens' k . q to its thread rows");
 
 __device__ __forceinline__ float delta_silu(float x) { return x / (1.0f + expf(-x)); }
 
@@ -86,6 +87,124 @@ __global__ __launch_bounds__(256) void delta_conv_kernel(const T* __restrict__ u
     }
 }
 
+// The same for runs of consecutive tokens: a wavefront walks `run` tokens of one unit with the taps and the last
+// J - 1 inputs of its elements in registers, so a token costs one new load per element whatever J (a workgroup a
+// token re-reads J rows and the taps for every token: 61 against 25 us for 2048 tokens of 4096 channels and four
+// taps).  Where the request changes inside a run the window is filled anew.
+template <typename T, int J>
+__global__ __launch_bounds__(256) void delta_conv_run_kernel(const T* __restrict__ u, int cols, const float* __restrict__ taps,
+                                                              const float* __restrict__ state, int64_t state_stride,
+                                                              const int32_t* __restrict__ token_seq,
+                                                              const int32_t* __restrict__ cu_tokens,
+                                                              const int32_t* __restrict__ seq_slots, float* __restrict__ q,
+                                                              float* __restrict__ k, float* __restrict__ v, int N, int run, int G,
+                                                              int dim, int H, int vdim, float unit_eps, float q_scale) {
+    constexpr int W = J > 1 ? J - 1 : 1;
+    const int unit = blockIdx.y * 4 + threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    if (unit >= 2 * G + H) return;
+    const int n0 = blockIdx.x * run, n1 = min(N, n0 + run);
+    int col0, width, out_cols, out0;
+    float* dst;
+    if (unit < G) {
+        col0 = unit * dim, width = dim, dst = q, out_cols = G * dim, out0 = unit * dim;
+    } else if (unit < 2 * G) {
+        col0 = unit * dim, width = dim, dst = k, out_cols = G * dim, out0 = (unit - G) * dim;
+    } else {
+        col0 = 2 * G * dim + (unit - 2 * G) * vdim, width = vdim, dst = v, out_cols = H * vdim, out0 = (unit - 2 * G) * vdim;
+    }
+    float tp[4][J], win[4][W];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int e = lane + LLE_WAVE * r;
+#pragma unroll
+        for (int j = 0; j < J; ++j) tp[r][j] = e < width ? taps[(int64_t)(col0 + e) * J + j] : 0.f;
+#pragma unroll
+        for (int m = 0; m < W; ++m) win[r][m] = 0.f;
+    }
+    int seq_before = -1;
+    for (int n = n0; n < n1; ++n) {
+        const int seq = token_seq[n];
+        if (J > 1 && seq != seq_before) {  // (the same for the whole wavefront) the J - 1 inputs ahead of this token
+            const int before = n - cu_tokens[seq];
+            const float* kept = state + (int64_t)seq_slots[seq] * state_stride;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int e = lane + LLE_WAVE * r;
+                if (e < width) {
+#pragma unroll
+                    for (int m = 0; m < W; ++m) {
+                        const int back = J - 1 - m;
+                        win[r][m] = back <= before ? to_f32<T>(u[(int64_t)(n - back) * cols + col0 + e])
+                                                   : kept[(int64_t)(J - 1 - (back - before)) * cols + col0 + e];
+                    }
+                }
+            }
+        }
+        seq_before = seq;
+        float y[4], ss = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int e = lane + LLE_WAVE * r;
+            y[r] = 0.f;
+            if (e < width) {
+                const float x = to_f32<T>(u[(int64_t)n * cols + col0 + e]);
+                float acc = 0.f;
+                if (J > 1) {
+#pragma unroll
+                    for (int m = 0; m < W; ++m) acc = fmaf(tp[r][m], win[r][m], acc);
+#pragma unroll
+                    for (int m = 0; m + 1 < W; ++m) win[r][m] = win[r][m + 1];
+                    win[r][W - 1] = x;
+                }
+                acc = fmaf(tp[r][J - 1], x, acc);
+                y[r] = delta_silu(acc);
+                ss = fmaf(y[r], y[r], ss);
+            }
+        }
+        float f = 1.0f;
+        if (unit < 2 * G) {
+            ss = wave_sum(ss);
+            f = 1.0f / sqrtf(ss + unit_eps);
+            if (unit < G) f *= q_scale;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int e = lane + LLE_WAVE * r;
+            if (e < width) dst[(int64_t)n * out_cols + out0 + e] = y[r] * f;
+        }
+    }
+}
+
+template <typename T>
+static bool delta_conv_runs(const void* u, int cols, const void* taps, int J, const void* state, int64_t state_stride,
+                            const void* token_seq, const void* cu_tokens, const void* seq_slots, void* q, void* k, void* v, int N,
+                            int G, int dim, int H, int vdim, float unit_eps, float q_scale, hipStream_t stream) {
+    const int blocks = (2 * G + H + 3) / 4;
+    // runs long enough that taps and windows are loaded seldom, short enough that a prompt fills the chip
+    int run = (int)((int64_t)N * blocks / 2048);
+    run = run < 1 ? 1 : run > 16 ? 16 : run;
+    const dim3 grid((N + run - 1) / run, blocks);
+#define DELTA_CONV_CASE(JJ)                                                                                                   \
+    case JJ:                                                                                                                  \
+        delta_conv_run_kernel<T, JJ><<<grid, 256, 0, stream>>>(                                                               \
+            (const T*)u, cols, (const float*)taps, (const float*)state, state_stride, (const int32_t*)token_seq,              \
+            (const int32_t*)cu_tokens, (const int32_t*)seq_slots, (float*)q, (float*)k, (float*)v, N, run, G, dim, H, vdim,   \
+            unit_eps, q_scale);                                                                                               \
+        return true;
+    switch (J) {
+        DELTA_CONV_CASE(1)
+        DELTA_CONV_CASE(2)
+        DELTA_CONV_CASE(3)
+        DELTA_CONV_CASE(4)
+        DELTA_CONV_CASE(5)
+        DELTA_CONV_CASE(6)
+        DELTA_CONV_CASE(7)
+        DELTA_CONV_CASE(8)
+    }
+#undef DELTA_CONV_CASE
+    return false;  // more taps: a workgroup a token
+}
+
 extern "C" int lle_delta_conv(const void* u, int cols, const void* taps, int J, const void* state, int64_t state_stride,
                               const void* token_seq, const void* cu_tokens, const void* seq_slots, void* q, void* k, void* v,
                               int N, int G, int dim, int H, int vdim, float unit_eps, float q_scale, int dtype,
@@ -94,6 +213,11 @@ extern "C" int lle_delta_conv(const void* u, int cols, const void* taps, int J, 
     if (J < 1 || (J > 1 && state == nullptr) || G <= 0 || H <= 0 || dim <= 0 || vdim <= 0 || dim > 4 * LLE_WAVE ||
         vdim > 4 * LLE_WAVE || cols != 2 * G * dim + H * vdim || (2 * G + H + 3) / 4 > 65535)
         return (int)hipErrorInvalidValue;
+    if (dtype == LLE_F32 ? delta_conv_runs<float>(u, cols, taps, J, state, state_stride, token_seq, cu_tokens, seq_slots, q, k, v, N, G,
+                                                  dim, H, vdim, unit_eps, q_scale, stream)
+                         : delta_conv_runs<bf16_t>(u, cols, taps, J, state, state_stride, token_seq, cu_tokens, seq_slots, q, k, v, N, G,
+                                                   dim, H, vdim, unit_eps, q_scale, stream))
+        LLE_RETURN_LAUNCH_STATUS();
     const dim3 grid(N, (2 * G + H + 3) / 4);
     if (dtype == LLE_F32)
         delta_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, cols, (const float*)taps, J, (const float*)state,
@@ -140,14 +264,70 @@ __device__ __forceinline__ float delta_row_sum(float x) {
     return x;
 }
 
+// What a thread reads of one staged token: its share of k and q, and the token's decay, beta and k . q.
+template <int KI>
+struct DeltaToken {
+    float kk[KI], qq[KI];
+    float g, beta, kq;
+};
+
+template <int KI>
+__device__ __forceinline__ void delta_read(DeltaToken<KI>& d, const float* __restrict__ kt, const float* __restrict__ qt,
+                                           const float4* __restrict__ par) {
+    if (KI % 4 == 0) {
+#pragma unroll
+        for (int ii = 0; ii < KI; ii += 4) {
+            const float4 a = *(const float4*)(kt + ii), b = *(const float4*)(qt + ii);
+            d.kk[ii] = a.x, d.kk[ii + 1] = a.y, d.kk[ii + 2] = a.z, d.kk[ii + 3] = a.w;
+            d.qq[ii] = b.x, d.qq[ii + 1] = b.y, d.qq[ii + 2] = b.z, d.qq[ii + 3] = b.w;
+        }
+    } else {
+#pragma unroll
+        for (int ii = 0; ii < KI; ++ii) {
+            d.kk[ii] = kt[ii];
+            d.qq[ii] = qt[ii];
+        }
+    }
+    const float4 pr = *par;
+    d.g = pr.x, d.beta = pr.y, d.kq = pr.z;
+}
+
+// One token of the walk for this thread's share of column j: both sums over the key channels in one pass, the
+// lanes' exchange, the correction; returns the read-out.
+template <int KI>
+__device__ __forceinline__ float delta_token(float (&S)[KI], const DeltaToken<KI>& d, float v) {
+    float p = 0.f, r = 0.f, gS[KI];
+#pragma unroll
+    for (int ii = 0; ii < KI; ++ii) {
+        p = fmaf(S[ii], d.kk[ii], p);
+        r = fmaf(S[ii], d.qq[ii], r);
+        gS[ii] = d.g * S[ii];
+    }
+    p = delta_row_sum(p);
+    r = delta_row_sum(r);
+    const float w = d.beta * fmaf(-d.g, p, v);
+#pragma unroll
+    for (int ii = 0; ii < KI; ++ii) S[ii] = fmaf(d.kk[ii], w, gS[ii]);
+    return fmaf(w, d.kq, d.g * r);
+}
+
 // grid = (requests, heads, blocks of DELTA_VB value channels).  Thread (jl, ig) = (tid / 16, tid % 16) owns the
-// key channels [ig KI, (ig + 1) KI) of column j = block DELTA_VB + jl.
+// key channels [ig KI, (ig + 1) KI) of column j = block DELTA_VB + jl.  The tokens pass through LDS DELTA_TC at a
+// time; the next chunk's q, k, v, beta and decay inputs are asked for before the current chunk is walked and wait
+// in registers meanwhile, and inside a chunk every token's operands leave LDS one token ahead of their use.
+// Measured at 2048 tokens of 32 heads of 64 x 64: everything asked for when it was needed 916 us; the next chunk
+// ahead and whole chunks without a condition per token 591 us; operands read a token ahead, decay, beta and k . q
+// in one 16-byte read 348 us.  Tried and not kept: all of a chunk's operands in registers before its first token
+// and k . q made in the walk (378 us, and two workgroups no longer share a CU: 194 against 116 us for four
+// requests of 512 tokens).
 template <int KI>
 __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) {
     constexpr int KD = KI * DELTA_IG;
+    constexpr int PER = DELTA_TC * KD / DELTA_THREADS;  // elements of q (and of k) of a chunk that a thread fetches
+    static_assert(DELTA_TC * KD % DELTA_THREADS == 0, "a chunk's q and k are dealt to the threads in equal shares");
     __shared__ __attribute__((aligned(16))) float s_q[DELTA_TC][KD];
     __shared__ __attribute__((aligned(16))) float s_k[DELTA_TC][KD];
-    __shared__ float s_g[DELTA_TC], s_beta[DELTA_TC], s_kq[DELTA_TC];
+    __shared__ float4 s_par[DELTA_TC];  // (decay, beta, k . q, -) of every staged token
     __shared__ float s_o[DELTA_TC][DELTA_VB];
     const int s = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, jl = tid / DELTA_IG, ig = tid % DELTA_IG;
@@ -163,59 +343,80 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
     for (int ii = 0; ii < KI; ++ii) S[ii] = (live && ig * KI + ii < dim) ? col[ii] : 0.f;
     const float decay_rate = expf(a.a_log[h]), dt_bias = a.dt_bias[h];
 
-    for (int c0 = q0; c0 < q1; c0 += DELTA_TC) {
-        const int nt = min(DELTA_TC, q1 - c0);
-        __syncthreads();  // (the chunk before has been read)
-        for (int idx = tid; idx < nt * KD; idx += DELTA_THREADS) {
-            const int t = idx / KD, i = idx - t * KD;
+    float fq[PER], fk[PER], fv[DELTA_TC], fb = 0.f, fa = 0.f;  // the chunk that is on its way
+    auto fetch = [&](int c0, int nt) {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
+            const bool there = t < nt && i < dim;
             const int64_t at = (int64_t)(c0 + t) * GD + hk * dim + i;
-            s_q[t][i] = i < dim ? a.q[at] : 0.f;
-            s_k[t][i] = i < dim ? a.k[at] : 0.f;
+            fq[r] = there ? a.q[at] : 0.f;
+            fk[r] = there ? a.k[at] : 0.f;
         }
+#pragma unroll
+        for (int t = 0; t < DELTA_TC; ++t) fv[t] = (t < nt && live) ? a.v[(int64_t)(c0 + t) * HV + h * vdim + j] : 0.f;
         if (tid < nt) {
             const float* ba = a.ba + (int64_t)(c0 + tid) * 2 * H;
-            const float x = ba[H + h] + dt_bias;
+            fb = ba[h];
+            fa = ba[H + h];
+        }
+    };
+    fetch(q0, min(DELTA_TC, q1 - q0));
+
+    for (int c0 = q0; c0 < q1; c0 += DELTA_TC) {
+        const int nt = min(DELTA_TC, q1 - c0);
+        __syncthreads();  // (the chunk before has been read, its results have left)
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
+            s_q[t][i] = fq[r];
+            s_k[t][i] = fk[r];
+        }
+        if (tid < nt) {
+            const float x = fa + dt_bias;
             const float softplus = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
-            s_beta[tid] = 1.0f / (1.0f + expf(-ba[h]));
-            s_g[tid] = expf(-decay_rate * softplus);
+            float* par = (float*)&s_par[tid];
+            par[0] = expf(-decay_rate * softplus);
+            par[1] = 1.0f / (1.0f + expf(-fb));
         }
         float vv[DELTA_TC];
 #pragma unroll
-        for (int t = 0; t < DELTA_TC; ++t) vv[t] = (t < nt && live) ? a.v[(int64_t)(c0 + t) * HV + h * vdim + j] : 0.f;
+        for (int t = 0; t < DELTA_TC; ++t) vv[t] = fv[t];
+        if (c0 + DELTA_TC < q1) fetch(c0 + DELTA_TC, min(DELTA_TC, q1 - c0 - DELTA_TC));
         __syncthreads();
-        {  // k . q of every token: a wavefront a token
-            const int wave = tid / LLE_WAVE, lane = tid % LLE_WAVE;
-            for (int t = wave; t < nt; t += DELTA_THREADS / LLE_WAVE) {
-                float d = 0.f;
-                for (int i = lane; i < KD; i += LLE_WAVE) d = fmaf(s_k[t][i], s_q[t][i], d);
-                d = wave_sum(d);
-                if (lane == 0) s_kq[t] = d;
-            }
+        {  // k . q of every token: the sixteen lanes of thread row jl take token jl (DELTA_VB == DELTA_TC)
+            float d = 0.f;
+            for (int i = ig; i < KD; i += DELTA_IG) d = fmaf(s_k[jl][i], s_q[jl][i], d);
+            d = delta_row_sum(d);
+            if (ig == 0) ((float*)&s_par[jl])[2] = d;
         }
         __syncthreads();
+        const float* kt = &s_k[0][ig * KI];
+        const float* qt = &s_q[0][ig * KI];
+        float oo[DELTA_TC];
+        if (nt == DELTA_TC) {  // a whole chunk: nothing under a condition, every token's operands read a token ahead
+            DeltaToken<KI> cur, nxt;
+            delta_read<KI>(cur, kt, qt, &s_par[0]);
 #pragma unroll
-        for (int t = 0; t < DELTA_TC; ++t) {
-            if (t < nt) {
-                float kk[KI], qq[KI];
-#pragma unroll
-                for (int ii = 0; ii < KI; ++ii) {
-                    kk[ii] = s_k[t][ig * KI + ii];
-                    qq[ii] = s_q[t][ig * KI + ii];
-                }
-                float p = 0.f, r = 0.f;
-#pragma unroll
-                for (int ii = 0; ii < KI; ++ii) {
-                    p = fmaf(S[ii], kk[ii], p);
-                    r = fmaf(S[ii], qq[ii], r);
-                }
-                p = delta_row_sum(p);
-                r = delta_row_sum(r);
-                const float g = s_g[t];
-                const float w = s_beta[t] * (vv[t] - g * p);
-#pragma unroll
-                for (int ii = 0; ii < KI; ++ii) S[ii] = fmaf(kk[ii], w, g * S[ii]);
-                if (ig == 0) s_o[t][jl] = fmaf(w, s_kq[t], g * r);
+            for (int t = 0; t < DELTA_TC; ++t) {
+                if (t + 1 < DELTA_TC) delta_read<KI>(nxt, kt + (t + 1) * KD, qt + (t + 1) * KD, &s_par[t + 1]);
+                oo[t] = delta_token<KI>(S, cur, vv[t]);
+                cur = nxt;
             }
+        } else {
+#pragma unroll
+            for (int t = 0; t < DELTA_TC; ++t) {
+                oo[t] = 0.f;
+                if (t < nt) {
+                    DeltaToken<KI> cur;
+                    delta_read<KI>(cur, kt + t * KD, qt + t * KD, &s_par[t]);
+                    oo[t] = delta_token<KI>(S, cur, vv[t]);
+                }
+            }
+        }
+        if (ig == 0) {
+#pragma unroll
+            for (int t = 0; t < DELTA_TC; ++t) s_o[t][jl] = oo[t];
         }
         __syncthreads();
         for (int idx = tid; idx < nt * DELTA_VB; idx += DELTA_THREADS) {

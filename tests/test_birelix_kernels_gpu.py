@@ -18,10 +18,13 @@ REF = TorchOps(torch.float64)
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("G,H,dim,vdim,J,q_lens", [(2, 6, 24, 20, 3, [5, 1, 1, 2]), (1, 1, 100, 12, 1, [7, 1]), (3, 3, 64, 256, 4, [1, 1, 1]),
-                                                   (2, 4, 256, 72, 6, [40, 3]), (1, 4, 8, 100, 2, [1, 9, 2])])
+                                                   (2, 4, 256, 72, 6, [40, 3]), (1, 4, 8, 100, 2, [1, 9, 2]), (1, 2, 16, 8, 9, [12, 1]),
+                                                   (16, 32, 8, 8, 4, [300, 1, 37, 2, 260])])
 def test_delta_convolution(dtype, G, H, dim, vdim, J, q_lens):
     """Single tokens, portions shorter and longer than the taps reach, state rows that are not zero and are
-    columns of a wider row; then the same tokens in smaller portions through the state give the same rows."""
+    columns of a wider row, more taps than the kernel for runs of tokens takes, and so many tokens that a
+    wavefront walks runs of them across the requests' borders; then the same tokens in smaller portions through
+    the state give the same rows."""
     o = ops()
     cols = 2 * G * dim + H * vdim
     seq_slots, cu, token_seq, N = batch(q_lens)
