@@ -11,7 +11,8 @@ import sys
 import pytest
 import torch
 
-from tests.birelix_util import CONFIGS, PAGE_SIZES, make_model_dir, plain_logits, read, residual_streams, run_tool, sharpen
+from tests.birelix_util import (CONFIGS, PAGE_SIZES, delta, dense, latent, layer, make_model_dir, moe, plain_logits, read,
+                                residual_streams, run_tool, sharpen, window)
 from tests.plain import birelix_plain as plain
 from tests.tiny import random_tokens
 from tests.trace_util import ROOT, TraceBuilder, changing_portions, check_dumps, mixed, tail_one_by_one, whole
@@ -53,6 +54,31 @@ def test_trace_gpu(tmp_path, which, dtype):
     run_tool(d, dtype, out, tb, page_size=None if default_page else PAGE_SIZES[which])
     worst = check_dumps(out, tb, plain_logits(d, requests), TOL[dtype])
     print(f"trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
+
+
+ONE_KIND = {
+    "delta": [layer("delta", delta(4, 2, 32, 24, 4), dense(40)), layer("delta", delta(2, 2, 64, 64, 2), None)],
+    "attention": [layer("attention", window(4, 2, 32, 32, 0.2, size=20), None), layer("attention", window(2, 1, 64, 48, 0.15), dense(40))],
+    "latent_attention": [layer("latent_attention", latent(4, 32, 16, 32, 64, 32, 0.15), None),
+                         layer("latent_attention", latent(2, 24, 8, 40, 48, 20, 0.2, 500.0), moe(4, 2, 24, 1.0, count=2, keep=1))],
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", list(ONE_KIND))
+def test_models_of_one_mixer_kind(tmp_path, kind, dtype):
+    """Delta layers alone (no pages at all), window attention alone, latent attention alone; a width and a vocabulary
+    that are multiples of two only."""
+    spec = {"architecture": "Birelix", "vocab": 90, "width": 76, "embedding": {"scale": 5.0}, "norm": {"eps": 1e-5},
+            "layers": ONE_KIND[kind]}
+    d = make_model_dir(tmp_path, kind, dtype=torch.bfloat16, config=spec)
+    sharpen(d, SHARP[dtype], same_experts=dtype == "bfloat16", skip=GENTLE[dtype])
+    requests = {rid: random_tokens(n, 90, 10 + i) for i, (rid, n) in enumerate(LENGTHS.items())}
+    tb = all_ways_trace(requests)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=16)
+    worst = check_dumps(out, tb, plain_logits(d, requests), TOL[dtype])
+    print(f"trace of {kind} alone, {dtype}: worst relative error {worst:.3g}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

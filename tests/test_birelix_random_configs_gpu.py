@@ -63,7 +63,7 @@ def draw_layer(rng):
 def draw(seed: int):
     rng = random.Random(seed)
     spec = {"architecture": "Birelix", "vocab": rng.choice([50, 97, 256, 311, 576]),
-            "width": rng.choice([64, 72, 96, 128, 136, 200, 256, 320]),
+            "width": rng.choice([64, 72, 96, 128, 136, 200, 256, 320, 52, 90]),
             "embedding": {"scale": rng.choice([1.0, 4.0, 8.0, 13.5])},
             "norm": {"eps": rng.choice([1e-6, 1e-5, 3e-6])}, "layers": [draw_layer(rng) for _ in range(rng.randint(2, 6))]}
     page = rng.choice([4, 8, 16, 16, 16, 32, 64])
