@@ -959,7 +959,7 @@ def birelix_config(which, groups):
     (W, LH, ldim, lrot, lvdim, rank, qrank, H, G, dim, vdim, window, DH, DG, ddim, dvdim, taps, E, top, eff, ng, keep, limit,
      ff) = BIRELIX_SIZES[which]
     lat = {"heads": LH, "dim": ldim, "rot_dim": lrot, "vdim": lvdim, "kv_rank": rank, "q_rank": qrank,
-           "scale": (ldim + lrot) ** -0.5, "rot": {"base": 250000.0, "dims": lrot}}
+           "scale": (ldim + lrot) ** -0.5, "rot": {"base": 10000.0, "dims": lrot}}
     att = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "mask": {"size": window}}
     dlt = {"heads": DH, "kv_heads": DG, "dim": ddim, "vdim": dvdim, "conv": taps}
     moe = {"kind": "moe", "expert": {"ff": eff, "limit": limit}, "router": {"experts": E, "top": top, "groups": {"count": ng, "keep": keep}}}

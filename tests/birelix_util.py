@@ -62,10 +62,10 @@ B_A = {
 B_B = {
     "architecture": "Birelix", "vocab": 256, "width": 128, "embedding": {"scale": 11.0}, "norm": {"eps": 1e-6},
     "layers": [
-        layer("latent_attention", latent(8, 32, 16, 32, 64, 48, 0.15, 250000.0), dense(96)),
-        layer("delta", delta(4, 2, 64, 32, 4), moe(8, 2, 32, 1.0, count=2, keep=1)),
+        layer("latent_attention", latent(8, 32, 16, 32, 64, 48, 0.15, 100000.0), dense(96)),
+        layer("delta", delta(4, 2, 64, 48, 3), moe(8, 3, 32, 1.5, count=2, keep=1)),
         layer("attention", window(8, 2, 64, 64, 0.12, size=48), moe(12, 3, 64, 3.0, count=4, keep=2)),
-        layer("latent_attention", latent(4, 64, 32, 64, 128, 96, 0.1, 10000.0), moe(8, 2, 32, 1.0, count=2, keep=1)),
+        layer("latent_attention", latent(4, 64, 32, 64, 128, 96, 0.1, 10000.0), moe(10, 2, 32, 1.0, count=5, keep=2)),
         layer("delta", delta(8, 8, 32, 64, 2), dense(64)),
         layer("attention", window(4, 4, 32, 32, 0.2), None),
     ],

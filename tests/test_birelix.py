@@ -144,14 +144,14 @@ def test_plain_latent_attention_written_out():
 
 
 def test_plain_router_groups_and_clamped_experts():
-    z = torch.tensor([2.0, -1.0, 0.5, 0.4, 0.3, 1.9, 1.0, 0.9], dtype=torch.float64)
+    z = torch.tensor([2.0, -1.0, 0.5, 0.3, 1.9, 1.0], dtype=torch.float64)
     s = plain.sigmoid(z)
-    # two groups of four, one kept: group 0 is worth s0 + s2, group 1 s5 + s6: group 1 wins although expert 0 is the best
+    # two groups of three, one kept: group 0 is worth s0 + s2, group 1 s4 + s5: group 1 wins although expert 0 is the best
     ids, weights = plain.router_choice(z, 2, 2, 1)
-    assert ids.tolist() == [5, 6] and torch.allclose(weights, s[[5, 6]] / s[[5, 6]].sum())
+    assert ids.tolist() == [4, 5] and torch.allclose(weights, s[[4, 5]] / s[[4, 5]].sum())
     ids, _ = plain.router_choice(z, 3, 2, 2)  # both kept: the three best of all
-    assert ids.tolist() == [0, 5, 6]
-    ids, weights = plain.router_choice(z, 1, 8, 3)  # groups of one expert: a group is worth its expert
+    assert ids.tolist() == [0, 4, 5]
+    ids, weights = plain.router_choice(z, 1, 6, 3)  # groups of one expert: a group is worth its expert
     assert ids.tolist() == [0] and abs(float(weights[0]) - 1.0) < 1e-12
     w = {"e.gate": rnd((3, 4), 1, 3.0), "e.up": rnd((3, 4), 2, 3.0), "e.down": rnd((4, 3), 3)}
     x = rnd((1, 4), 4)

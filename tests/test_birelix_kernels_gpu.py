@@ -177,7 +177,7 @@ def test_latent_attention_without_a_sink(dtype, P, rank, rot, H, lens, pasts):
 
 
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("E,top,groups,keep,group_top", [(12, 4, 4, 3, 2), (8, 2, 2, 1, 2), (70, 5, 7, 2, 3), (6, 1, 6, 1, 2), (64, 6, 8, 8, 2),
+@pytest.mark.parametrize("E,top,groups,keep,group_top", [(12, 4, 4, 3, 2), (10, 3, 2, 1, 2), (70, 5, 7, 2, 3), (6, 1, 6, 1, 2), (64, 6, 8, 8, 2),
                                                          (9, 3, 3, 2, 1)])
 def test_sigmoid_router_with_groups_worth_their_largest_scores(E, top, groups, keep, group_top):
     o = ops()
@@ -191,10 +191,10 @@ def test_sigmoid_router_with_groups_worth_their_largest_scores(E, top, groups, k
 
 def test_sigmoid_router_a_group_of_two_good_experts_beats_the_group_of_the_best_and_ties():
     o = ops()
-    z = torch.tensor([[2.0, -1.0, 0.5, 0.4, 0.3, 1.9, 1.0, 0.9]]).cuda()
+    z = torch.tensor([[2.0, -1.0, 0.5, 0.3, 1.9, 1.0]]).cuda()
     ids, gains = o.moe_route_grouped(z, None, 2, 2, 1, score="sigmoid", group_top=2)
-    assert ids.tolist() == [[5, 6]]
-    s = torch.sigmoid(z[0, [5, 6]])
+    assert ids.tolist() == [[4, 5]]
+    s = torch.sigmoid(z[0, [4, 5]])
     assert (gains[0] - s / s.sum()).abs().max() < 1e-6
     ids, _ = o.moe_route_grouped(z, None, 2, 2, 1, score="sigmoid", group_top=1)  # by their best expert alone: group 0
     assert ids.tolist() == [[0, 2]]

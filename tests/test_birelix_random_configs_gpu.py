@@ -36,12 +36,12 @@ def draw_layer(rng):
         dim, rot = rng.choice([8, 16, 32, 64, 128]), rng.choice([2, 6, 8, 16, 32, 64])
         mixer = latent(rng.choice([1, 2, 3, 8, 16]), dim, rot, rng.choice([8, 24, 32, 64, 128]), rng.choice([8, 16, 40, 64, 128, 160]),
                        rng.choice([6, 16, 48, 96]), round(rng.choice([0.7, 1.0, 1.4]) / (dim + rot) ** 0.5, 4),
-                       rng.choice([50.0, 1e4, 2.5e5]), dims=rng.choice([rot, rot, 2, rot // 4 * 2 or 2]))
+                       rng.choice([50.0, 1e4, 1e5]), dims=rng.choice([rot, rot, 2, rot // 4 * 2 or 2]))
     elif kind == "attention":
         dim = rng.choice([16, 32, 48, 64, 64, 96, 128, 256])
         nkv = rng.choice([1, 1, 2, 3, 4])
         mixer = window(nkv * rng.choice([1, 2, 3, 4, 8]), nkv, dim, rng.choice([dim, dim, 16, 32, 64, 80, 256]),
-                       round(rng.choice([0.7, 1.0, 1.4]) / dim ** 0.5, 4), rng.choice([None, 1, 2, 7, 16, 33, 64, 72, 200]))
+                       round(rng.choice([0.7, 1.0, 1.4]) / dim ** 0.5, 4), rng.choice([None, 1, 2, 7, 16, 33, 64, 70, 200]))
     else:
         nkv = rng.choice([1, 1, 2, 3, 4])
         mixer = delta(nkv * rng.choice([1, 1, 2, 3, 4]), nkv, rng.choice([8, 16, 24, 32, 64, 64, 100, 128, 256]),
