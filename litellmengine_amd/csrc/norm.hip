@@ -300,10 +300,10 @@ extern "C" int lle_add_rmsnorm(void* hidden, const void* delta, const void* rows
     LLE_RETURN_LAUNCH_STATUS();
 }
 
-// plain RMSNorm of activation rows x [R, H] of type T (no residual): out = norm(x) * w
-template <typename T>
+// plain RMSNorm of activation rows x [R, H] of type T (no residual): out = norm(x) * w, in the type TO
+template <typename T, typename TO = T>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const void* __restrict__ weight,
-                                                       int weight_dtype, T* __restrict__ out, int H, float eps) {
+                                                       int weight_dtype, TO* __restrict__ out, int H, float eps) {
     __shared__ float red[16];
     const int64_t r = blockIdx.x;
     const T* xr = x + r * H;
@@ -314,9 +314,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, c
     }
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-    T* o = out + r * H;
+    TO* o = out + r * H;
     for (int i = threadIdx.x; i < H; i += blockDim.x)
-        o[i] = from_f32<T>(to_f32<T>(xr[i]) * inv * load_as_f32(weight, i, weight_dtype));
+        o[i] = from_f32<TO>(to_f32<T>(xr[i]) * inv * load_as_f32(weight, i, weight_dtype));
 }
 
 extern "C" int lle_rmsnorm(const void* x, const void* weight, int weight_dtype, void* out, int R, int H, float eps,
@@ -326,6 +326,14 @@ extern "C" int lle_rmsnorm(const void* x, const void* weight, int weight_dtype, 
         rmsnorm_kernel<float><<<R, 256, 0, stream>>>((const float*)x, weight, weight_dtype, (float*)out, H, eps);
     else
         rmsnorm_kernel<bf16_t><<<R, 256, 0, stream>>>((const bf16_t*)x, weight, weight_dtype, (bf16_t*)out, H, eps);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// float32 rows in, bfloat16 rows out: the norm of a product's 32-bit result, handed on in the activation type
+extern "C" int lle_rmsnorm_f32_to_bf16(const void* x, const void* weight, int weight_dtype, void* out, int R, int H, float eps,
+                                       hipStream_t stream) {
+    if (R <= 0) return 0;
+    rmsnorm_kernel<float, bf16_t><<<R, 256, 0, stream>>>((const float*)x, weight, weight_dtype, (bf16_t*)out, H, eps);
     LLE_RETURN_LAUNCH_STATUS();
 }
 

@@ -186,12 +186,19 @@ class HipOps:
                   R, H, float(eps), dtype_code(out_dtype))
         return out
 
-    def rmsnorm(self, x, weight, eps: float) -> torch.Tensor:
-        """x [R, H] -> x * rsqrt(mean(x^2) + eps) * weight, same type."""
+    def rmsnorm(self, x, weight, eps: float, out_dtype=None) -> torch.Tensor:
+        """x [R, H] -> x * rsqrt(mean(x^2) + eps) * weight, same type (`out_dtype` bfloat16 for float32 rows: the
+        result in bfloat16 from the same launch)."""
         _dev(x, "x")
         _dev(weight, "norm weight")
         R, H = x.shape
         _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        if out_dtype is not None and out_dtype != x.dtype:
+            _need(x.dtype == torch.float32 and out_dtype == torch.bfloat16, "a norm hands float32 rows on as they are or in bfloat16")
+            out = torch.empty((R, H), dtype=out_dtype, device=x.device)
+            self._run("norm", "lle_rmsnorm_f32_to_bf16", [_P, _P, _I, _P, _I, _I, _F, _P],
+                      _ptr(x), _ptr(weight), dtype_code(weight.dtype), _ptr(out), R, H, float(eps))
+            return out
         out = torch.empty_like(x)
         self._run("norm", "lle_rmsnorm", [_P, _P, _I, _P, _I, _I, _F, _I, _P],
                   _ptr(x), _ptr(weight), dtype_code(weight.dtype), _ptr(out), R, H, float(eps), dtype_code(x.dtype))

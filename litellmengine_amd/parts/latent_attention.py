@@ -115,8 +115,8 @@ class LatentAttention(Mixer):
         if self.dq is None:
             q = self.q.forward(x)
         else:  # the queries' latent: its norm reads the product's 32-bit result
-            cq = ops.rmsnorm(self.dq.forward(x, out_dtype=torch.float32), self.q_norm_w, self.eps)
-            q = self.q.forward(ops.cast(cq, self.ctx.dtype))
+            q = self.q.forward(ops.rmsnorm(self.dq.forward(x, out_dtype=torch.float32), self.q_norm_w, self.eps,
+                                           out_dtype=self.ctx.dtype))
         dkv = self.dkv.forward(x)
         if cache.writes:
             ops.latent_kv_write(dkv, self.norm_w, self.eps, cos_sin, rot_dims, group.slot_mapping, cache.pages,

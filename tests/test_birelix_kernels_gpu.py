@@ -176,6 +176,27 @@ def test_latent_attention_without_a_sink(dtype, P, rank, rot, H, lens, pasts):
     assert (got[0].float() - one["pages"][page, :rank].float()).abs().max() < tol(dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES + ["bfloat16 queries"])
+@pytest.mark.parametrize("far", [3, 15, 16, 597])
+def test_latent_attention_without_a_sink_one_key_among_hundreds(dtype, far):
+    """One key (near the start, on both sides of a page's border, near the end) is made to carry the softmax of a
+    decoded token after 600 others: the result is that key's latent row."""
+    o = ops()
+    P, rank, rot, H = 16, 64, 8, 2
+    q_dtype = torch.float32 if dtype != "bfloat16 queries" else torch.bfloat16  # (the latter: the matrix-core kernel)
+    dtype = torch.bfloat16 if dtype == "bfloat16 queries" else dtype
+    c = latent_case(dtype, P, rank, rot, H, [1], [600], 31)
+    page = int(c["table"][int(c["seq_slots"][0]), far // P])
+    row = c["pages"][page, (far % P) * rank : (far % P + 1) * rank].float()
+    q_lat = (row * 40.0 / (row * row).sum()).view(1, 1, rank).repeat(1, H, 1).contiguous().to(q_dtype)
+    q_rot = torch.zeros((1, H, rot), dtype=torch.float32).cuda()
+    args = [q_lat, q_rot, c["pages"], P, rank, rot, c["table"], c["seq_slots"], c["cu"], c["kv_lens"], c["token_seq"], None,
+            None, 1.0, 1, 601, dtype]
+    got = o.latent_attention(*args)
+    assert (got.double() - REF.latent_attention(*args).double()).abs().max() < tol(dtype)
+    assert (got[0, 0].float() - row).abs().max() < 0.05 and (got[0, 1].float() - row).abs().max() < 0.05
+
+
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("E,top,groups,keep,group_top", [(12, 4, 4, 3, 2), (10, 3, 2, 1, 2), (70, 5, 7, 2, 3), (6, 1, 6, 1, 2), (64, 6, 8, 8, 2),
                                                          (9, 3, 3, 2, 1)])
@@ -220,6 +241,18 @@ def test_clamped_experts(dtype, N, K, F, H, E, top, limit):
     assert (got.double() - want.double()).abs().max() < tol(dtype, 4)
     unclamped = REF.moe_experts(x, ids, gains, gate_up, down, form="gated_clamp", limit=1e9)
     assert (unclamped.double() - want.double()).abs().max() > 0.05
+
+
+@pytest.mark.parametrize("H", [6, 80, 1536])
+def test_norm_of_32_bit_rows_handed_on_in_bfloat16(H):
+    o = ops()
+    x = rnd((9, H), torch.float32, 1, 3.0)
+    w = (1.0 + rnd((H,), torch.float32, 2, 0.1)).to(torch.bfloat16)
+    got = o.rmsnorm(x, w, 1e-5, out_dtype=torch.bfloat16)
+    want = REF.rmsnorm(x, w, 1e-5, out_dtype=torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and (got.double() - want.double()).abs().max() < tol(torch.bfloat16, 4)
+    same = o.rmsnorm(x, w, 1e-5, out_dtype=torch.float32)
+    assert same.dtype == torch.float32 and (same.double() - REF.rmsnorm(x, w, 1e-5).double()).abs().max() < 1e-5
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

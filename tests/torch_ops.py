@@ -62,10 +62,10 @@ class TorchOps:
         y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(self.cd)
         return y.to(out_dtype)
 
-    def rmsnorm(self, x, weight, eps):
+    def rmsnorm(self, x, weight, eps, out_dtype=None):
         xx = x.to(self.cd)
         y = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(self.cd)
-        return y.to(x.dtype)
+        return y.to(out_dtype or x.dtype)
 
     def linear(self, x, weight, out_dtype=None, fold=None, sums_ok=False):
         assert fold is None, "this stand-in folds no norm (can_fold_norm says so)"
