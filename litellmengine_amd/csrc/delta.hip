@@ -317,7 +317,8 @@ __device__ __forceinline__ float delta_token(float (&S)[KI], const DeltaToken<KI
 // in registers meanwhile, and inside a chunk every token's operands leave LDS one token ahead of their use.
 // Measured at 2048 tokens of 32 heads of 64 x 64: everything asked for when it was needed 916 us; the next chunk
 // ahead and whole chunks without a condition per token 591 us; operands read a token ahead, decay, beta and k . q
-// in one 16-byte read 348 us.  Tried and not kept: all of a chunk's operands in registers before its first token
+// in one 16-byte read 348 us; the chunk's values through LDS, one load a thread 294 us; q and k staged 16 bytes at a
+// time 281 us.  Tried and not kept: all of a chunk's operands in registers before its first token
 // and k . q made in the walk (378 us, and two workgroups no longer share a CU: 194 against 116 us for four
 // requests of 512 tokens).
 template <int KI>
@@ -329,6 +330,7 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
     __shared__ __attribute__((aligned(16))) float s_k[DELTA_TC][KD];
     __shared__ float4 s_par[DELTA_TC];  // (decay, beta, k . q, -) of every staged token
     __shared__ float s_o[DELTA_TC][DELTA_VB];
+    __shared__ float s_v[DELTA_TC][DELTA_VB];
     const int s = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, jl = tid / DELTA_IG, ig = tid % DELTA_IG;
     const int j0 = blockIdx.z * DELTA_VB, j = j0 + jl;
@@ -343,18 +345,37 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
     for (int ii = 0; ii < KI; ++ii) S[ii] = (live && ig * KI + ii < dim) ? col[ii] : 0.f;
     const float decay_rate = expf(a.a_log[h]), dt_bias = a.dt_bias[h];
 
-    float fq[PER], fk[PER], fv[DELTA_TC], fb = 0.f, fa = 0.f;  // the chunk that is on its way
+    float fq[PER], fk[PER], fv = 0.f, fb = 0.f, fa = 0.f;  // the chunk that is on its way
+    const bool wide = PER % 4 == 0 && dim == KD;  // whole heads of a multiple of 64 channels: 16 bytes a load and a store
     auto fetch = [&](int c0, int nt) {
+        if (wide) {
 #pragma unroll
-        for (int r = 0; r < PER; ++r) {
-            const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
-            const bool there = t < nt && i < dim;
-            const int64_t at = (int64_t)(c0 + t) * GD + hk * dim + i;
-            fq[r] = there ? a.q[at] : 0.f;
-            fk[r] = there ? a.k[at] : 0.f;
+            for (int r = 0; r + 3 < PER; r += 4) {
+                const int e = (tid + DELTA_THREADS * (r / 4)) * 4, t = e / KD, i = e - t * KD;
+                float4 x = float4{0.f, 0.f, 0.f, 0.f}, y = x;
+                if (t < nt) {
+                    const int64_t at = (int64_t)(c0 + t) * GD + hk * dim + i;
+                    x = *(const float4*)(a.q + at);
+                    y = *(const float4*)(a.k + at);
+                }
+                fq[r] = x.x, fq[r + 1] = x.y, fq[r + 2] = x.z, fq[r + 3] = x.w;
+                fk[r] = y.x, fk[r + 1] = y.y, fk[r + 2] = y.z, fk[r + 3] = y.w;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
+                const bool there = t < nt && i < dim;
+                const int64_t at = (int64_t)(c0 + t) * GD + hk * dim + i;
+                fq[r] = there ? a.q[at] : 0.f;
+                fk[r] = there ? a.k[at] : 0.f;
+            }
         }
-#pragma unroll
-        for (int t = 0; t < DELTA_TC; ++t) fv[t] = (t < nt && live) ? a.v[(int64_t)(c0 + t) * HV + h * vdim + j] : 0.f;
+        {  // the chunk's values of the workgroup's columns: one element a thread (one load a lane and token, sixteen
+           // lanes asking for the same word, kept the memory pipeline busy for longer than the walk itself)
+            const int t = tid / DELTA_VB, e = tid % DELTA_VB;
+            fv = (t < nt && j0 + e < vdim) ? a.v[(int64_t)(c0 + t) * HV + h * vdim + j0 + e] : 0.f;
+        }
         if (tid < nt) {
             const float* ba = a.ba + (int64_t)(c0 + tid) * 2 * H;
             fb = ba[h];
@@ -366,11 +387,20 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
     for (int c0 = q0; c0 < q1; c0 += DELTA_TC) {
         const int nt = min(DELTA_TC, q1 - c0);
         __syncthreads();  // (the chunk before has been read, its results have left)
+        if (wide) {
 #pragma unroll
-        for (int r = 0; r < PER; ++r) {
-            const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
-            s_q[t][i] = fq[r];
-            s_k[t][i] = fk[r];
+            for (int r = 0; r + 3 < PER; r += 4) {
+                const int e = (tid + DELTA_THREADS * (r / 4)) * 4, t = e / KD, i = e - t * KD;
+                *(float4*)&s_q[t][i] = float4{fq[r], fq[r + 1], fq[r + 2], fq[r + 3]};
+                *(float4*)&s_k[t][i] = float4{fk[r], fk[r + 1], fk[r + 2], fk[r + 3]};
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const int e = tid + DELTA_THREADS * r, t = e / KD, i = e - t * KD;
+                s_q[t][i] = fq[r];
+                s_k[t][i] = fk[r];
+            }
         }
         if (tid < nt) {
             const float x = fa + dt_bias;
@@ -379,11 +409,12 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
             par[0] = expf(-decay_rate * softplus);
             par[1] = 1.0f / (1.0f + expf(-fb));
         }
-        float vv[DELTA_TC];
-#pragma unroll
-        for (int t = 0; t < DELTA_TC; ++t) vv[t] = fv[t];
+        s_v[tid / DELTA_VB][tid % DELTA_VB] = fv;
         if (c0 + DELTA_TC < q1) fetch(c0 + DELTA_TC, min(DELTA_TC, q1 - c0 - DELTA_TC));
         __syncthreads();
+        float vv[DELTA_TC];
+#pragma unroll
+        for (int t = 0; t < DELTA_TC; ++t) vv[t] = s_v[t][jl];
         {  // k . q of every token: the sixteen lanes of thread row jl take token jl (DELTA_VB == DELTA_TC)
             float d = 0.f;
             for (int i = ig; i < KD; i += DELTA_IG) d = fmaf(s_k[jl][i], s_q[jl][i], d);
