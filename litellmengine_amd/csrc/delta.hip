@@ -248,7 +248,23 @@ struct DeltaArgs {
     const int32_t* cu_tokens;
     float* out;            // [N, H vdim]
     int H, G, dim, vdim;
+    const float* gates;    // [N, 2 H]: decay and beta of every token and head, made ahead (or null: made in the walk)
 };
+
+// decay and beta of every token and head, for the walks of long portions: in the walk itself the exponentials and the
+// logarithm of a chunk's sixteen tokens are one wavefront's work while the other three wait (a ninth of the walk's time)
+__global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restrict__ ba, const float* __restrict__ a_log,
+                                                           const float* __restrict__ dt_bias, float* __restrict__ gates,
+                                                           int64_t total, int H) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t n = idx / H;
+    const int h = (int)(idx - n * H);
+    const float x = ba[n * 2 * H + H + h] + dt_bias[h];
+    const float softplus = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
+    gates[n * 2 * H + h] = expf(-expf(a_log[h]) * softplus);
+    gates[n * 2 * H + H + h] = 1.0f / (1.0f + expf(-ba[n * 2 * H + h]));
+}
 
 template <int CTRL>
 __device__ __forceinline__ float delta_lanes(float x) {  // x of the lane that the pattern names
@@ -318,7 +334,7 @@ __device__ __forceinline__ float delta_token(float (&S)[KI], const DeltaToken<KI
 // Measured at 2048 tokens of 32 heads of 64 x 64: everything asked for when it was needed 916 us; the next chunk
 // ahead and whole chunks without a condition per token 591 us; operands read a token ahead, decay, beta and k . q
 // in one 16-byte read 348 us; the chunk's values through LDS, one load a thread 294 us; q and k staged 16 bytes at a
-// time 281 us.  Tried and not kept: all of a chunk's operands in registers before its first token
+// time 281 us; decays and betas made by a launch ahead of the walk 248 us.  Tried and not kept: all of a chunk's operands in registers before its first token
 // and k . q made in the walk (378 us, and two workgroups no longer share a CU: 194 against 116 us for four
 // requests of 512 tokens).
 template <int KI>
@@ -376,10 +392,10 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
             const int t = tid / DELTA_VB, e = tid % DELTA_VB;
             fv = (t < nt && j0 + e < vdim) ? a.v[(int64_t)(c0 + t) * HV + h * vdim + j0 + e] : 0.f;
         }
-        if (tid < nt) {
-            const float* ba = a.ba + (int64_t)(c0 + tid) * 2 * H;
-            fb = ba[h];
-            fa = ba[H + h];
+        if (tid < nt) {  // (with gates made ahead: beta, then the decay itself)
+            const float* ba = (a.gates ? a.gates : a.ba) + (int64_t)(c0 + tid) * 2 * H;
+            fb = a.gates ? ba[H + h] : ba[h];
+            fa = a.gates ? ba[h] : ba[H + h];
         }
     };
     fetch(q0, min(DELTA_TC, q1 - q0));
@@ -403,11 +419,16 @@ __global__ __launch_bounds__(DELTA_THREADS) void delta_scan_kernel(DeltaArgs a) 
             }
         }
         if (tid < nt) {
-            const float x = fa + dt_bias;
-            const float softplus = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
             float* par = (float*)&s_par[tid];
-            par[0] = expf(-decay_rate * softplus);
-            par[1] = 1.0f / (1.0f + expf(-fb));
+            if (a.gates) {
+                par[0] = fa;
+                par[1] = fb;
+            } else {
+                const float x = fa + dt_bias;
+                const float softplus = fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
+                par[0] = expf(-decay_rate * softplus);
+                par[1] = 1.0f / (1.0f + expf(-fb));
+            }
         }
         s_v[tid / DELTA_VB][tid % DELTA_VB] = fv;
         if (c0 + DELTA_TC < q1) fetch(c0 + DELTA_TC, min(DELTA_TC, q1 - c0 - DELTA_TC));
@@ -466,15 +487,21 @@ extern "C" int lle_delta_max_dim(void) { return 16 * DELTA_IG; }
 
 // q, k float32 [N, G dim] (unit vectors, q scaled), v float32 [N, H vdim], ba float32 [N, 2 H], a_log and dt_bias
 // float32 [H]; state float32 rows of `state_stride` floats whose first H vdim dim hold the heads' states transposed;
-// out float32 [N, H vdim]
+// out float32 [N, H vdim]; `gates` (or null) scratch float32 [N, 2 H] for the decays and betas made ahead of the walk
 extern "C" int lle_delta_scan(const void* q, const void* k, const void* v, const void* ba, const void* a_log,
                               const void* dt_bias, void* state, int64_t state_stride, const void* seq_slots,
-                              const void* cu_tokens, void* out, int S, int H, int G, int dim, int vdim, hipStream_t stream) {
+                              const void* cu_tokens, void* out, int S, int H, int G, int dim, int vdim, void* gates, int N,
+                              hipStream_t stream) {
     if (S <= 0 || H <= 0) return 0;
     if (G <= 0 || H % G || dim <= 0 || dim > 16 * DELTA_IG || vdim <= 0 || H > 65535 || (vdim + DELTA_VB - 1) / DELTA_VB > 65535)
         return (int)hipErrorInvalidValue;
     DeltaArgs a{(const float*)q, (const float*)k, (const float*)v, (const float*)ba, (const float*)a_log, (const float*)dt_bias,
-                (float*)state, state_stride, (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (float*)out, H, G, dim, vdim};
+                (float*)state, state_stride, (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (float*)out, H, G, dim, vdim, (const float*)gates};
+    if (gates != nullptr) {  // scratch float32 [N, 2 H], given for steps with long portions
+        const int64_t total = (int64_t)N * H;
+        delta_gates_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>((const float*)ba, (const float*)a_log,
+                                                                            (const float*)dt_bias, (float*)gates, total, H);
+    }
     const dim3 grid(S, H, (vdim + DELTA_VB - 1) / DELTA_VB);
 #define DELTA_CASE(KI)                                                      \
     if (dim <= KI * DELTA_IG) {                                             \

@@ -1309,6 +1309,8 @@ class HipOps:
                   float(unit_eps), float(q_scale), dtype_code(u.dtype))
         return q, k, v
 
+    DELTA_GATES_AHEAD = 64  # tokens of a step from which decays and betas are made by a launch of their own
+
     def delta_scan(self, q, k, v, ba, a_log, dt_bias, state, heads: int, kv_heads: int, dim: int, vdim: int, seq_slots,
                    cu_tokens) -> torch.Tensor:
         """Per head h, with the matrix state S [dim, vdim] of the request (float32; `state[slot]` holds the heads'
@@ -1333,9 +1335,12 @@ class HipOps:
         _need(state.shape[1] >= H * vdim * dim, "a state row holds heads * vdim * dim floats")
         _need(cu_tokens.shape == (S + 1,), "cu_tokens must be [S + 1]")
         out = torch.empty((N, H * vdim), dtype=torch.float32, device=v.device)
-        self._run("delta", "lle_delta_scan", [_P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+        # steps with portions: the exponentials of decay and beta leave the walk (a step of single tokens keeps them there:
+        # one launch less).  The number of tokens is known on the host and fixed inside a graph.
+        gates = torch.empty((N, 2 * H), dtype=torch.float32, device=v.device) if N >= max(self.DELTA_GATES_AHEAD, 2 * S) else None
+        self._run("delta", "lle_delta_scan", [_P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _P],
                   _ptr(q), _ptr(k), _ptr(v), _ptr(ba), _ptr(a_log), _ptr(dt_bias), _ptr(state), state.stride(0),
-                  _ptr(seq_slots), _ptr(cu_tokens), _ptr(out), S, H, G, dim, vdim)
+                  _ptr(seq_slots), _ptr(cu_tokens), _ptr(out), S, H, G, dim, vdim, _ptr(gates), N)
         return out
 
     def delta_out_norm(self, o, gate, norm_w, eps: float, heads: int, vdim: int) -> torch.Tensor:

@@ -56,10 +56,11 @@ def test_delta_convolution(dtype, G, H, dim, vdim, J, q_lens):
 
 @pytest.mark.parametrize("H,G,dim,vdim,q_lens", [(6, 2, 24, 20, [5, 1, 1, 30]), (1, 1, 100, 12, [17, 1]), (4, 4, 64, 64, [1, 1, 1]),
                                                  (2, 1, 256, 40, [70]), (4, 1, 8, 100, [3, 9]), (3, 3, 128, 16, [1, 26]),
-                                                 (2, 2, 16, 33, [12, 1])])
+                                                 (2, 2, 16, 33, [12, 1]), (4, 2, 32, 24, [40, 1, 33, 2])])
 def test_delta_walk(H, G, dim, vdim, q_lens):
-    """From states that are not zero, portions beside single tokens; then a portion cut in pieces gives the same
-    rows and the same state as in one go."""
+    """From states that are not zero, portions beside single tokens (steps of many tokens make decays and betas in
+    a launch ahead of the walk, short ones in the walk); then a portion cut in pieces gives the same rows and the
+    same state as in one go."""
     o = ops()
     seq_slots, cu, token_seq, N = batch(q_lens)
     unit = lambda t, heads: torch.nn.functional.normalize(t.view(N, heads, dim), dim=-1).reshape(N, heads * dim).contiguous()
